@@ -1,0 +1,230 @@
+"""ctypes front end of the CPU oracle (libzkoracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py.  The product (the HIP library and its `kernel`
+module) never imports this file.
+
+All functions take and return C-contiguous numpy arrays and mirror the Python
+operator API of the reference's inference/kernel.py:341-688 (same argument
+order and meaning), except that nothing lives on a GPU.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libzkoracle.so")
+
+
+def build(force=False):
+    """Compile libzkoracle.so with gcc (a second or two)."""
+    src = os.path.join(_HERE, "zk_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libzkoracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+def _load():
+    if not os.path.exists(_SO):
+        build()
+    lib = ctypes.CDLL(_SO)
+    vp, ll, ci, cl = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_long
+    for name in ("ora_int64_64_bmm_broadcast", "ora_int64_32_bmm_broadcast"):
+        getattr(lib, name).argtypes = [vp, vp, vp, vp, ll, ll, ll, ci, ci, ci, ci]
+    for name in ("ora_einsum_bshd_hdc_bshc", "ora_einsum_bshc_btc_bsht",
+                 "ora_einsum_bsht_btc_bshc", "ora_einsum_bshc_hdc_bshd"):
+        getattr(lib, name).argtypes = [vp, vp, vp, ll, ci, ci, ci, ci, ci]
+    lib.ora_complex_int64_mul.argtypes = [vp, vp, vp, ci, ci, ci, ci]
+    lib.ora_rms_stat.argtypes = [vp, vp, ci, ci, ll, ll]
+    lib.ora_rms_stat.restype = ci
+    lib.ora_rms_norm_32.argtypes = [vp, vp, vp, vp, ci, ci]
+    lib.ora_rms_norm_64.argtypes = [vp, vp, vp, vp, ci, ci]
+    for name in ("ora_softmax_init_q19", "ora_softmax_init_q21", "ora_silu_init_q23", "ora_silu_init_q25"):
+        getattr(lib, name).argtypes = [vp]
+    for name in ("ora_softmax_q19", "ora_softmax_q21"):
+        getattr(lib, name).argtypes = [vp, vp, vp, vp, ci, ci, ci, ci]
+    for name in ("ora_act_q23", "ora_act_q25"):
+        getattr(lib, name).argtypes = [vp, vp, vp, cl, ci]
+    lib.ora_set_threads.argtypes = [ci]
+    lib.ora_max_threads.restype = ci
+    return lib
+
+
+_lib = _load()
+
+
+def set_threads(n):
+    _lib.ora_set_threads(int(n))
+
+
+def max_threads():
+    return int(_lib.ora_max_threads())
+
+
+def _c(a, dtype=np.int64):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == dtype, (a.dtype, dtype)
+    return a
+
+
+def _p(a):
+    return a.ctypes.data
+
+
+def int64_bmm_broadcast(A, B, a_rescale, b_rescale, c_rescale):
+    """(C, R) of inference/kernel.py:341-371."""
+    A = _c(A)
+    Bdim, M, K = A.shape
+    N, K2 = B.shape
+    assert K2 == K
+    C = np.empty((Bdim, M, N), np.int64)
+    R = np.empty((Bdim, M, N), np.int64)
+    if B.dtype == np.int64:
+        B = _c(B)
+        _lib.ora_int64_64_bmm_broadcast(_p(A), _p(B), _p(C), _p(R), a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
+    else:
+        B = _c(B, np.int32)
+        _lib.ora_int64_32_bmm_broadcast(_p(A), _p(B), _p(C), _p(R), a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
+    return C, R
+
+
+def einsum_bshd_hdc_bshc(A, B, rescale):
+    A, B = _c(A), _c(B, np.int32)
+    Bt, S, H, D = A.shape
+    assert B.shape[0] == H and B.shape[1] == D
+    Cp = B.shape[2]
+    out = np.empty((Bt, S, H, Cp), np.int64)
+    _lib.ora_einsum_bshd_hdc_bshc(_p(A), _p(B), _p(out), rescale, Bt, S, H, D, Cp)
+    return out
+
+
+def einsum_bshc_btc_bsht(A, B, rescale):
+    A, B = _c(A), _c(B)
+    Bsz, S, H, Cdim = A.shape
+    T = B.shape[1]
+    assert B.shape[0] == Bsz and B.shape[2] == Cdim
+    out = np.empty((Bsz, S, H, T), np.int64)
+    _lib.ora_einsum_bshc_btc_bsht(_p(A), _p(B), _p(out), rescale, Bsz, S, H, T, Cdim)
+    return out
+
+
+def einsum_bsht_btc_bshc(A, B, rescale):
+    A, B = _c(A), _c(B)
+    Bsz, S, H, T = A.shape
+    Cdim = B.shape[2]
+    assert B.shape[0] == Bsz and B.shape[1] == T
+    out = np.empty((Bsz, S, H, Cdim), np.int64)
+    _lib.ora_einsum_bsht_btc_bshc(_p(A), _p(B), _p(out), rescale, Bsz, S, H, T, Cdim)
+    return out
+
+
+def einsum_bshc_hdc_bshd(A, B, rescale):
+    A, B = _c(A), _c(B, np.int32)
+    Bsz, S, H, Cdim = A.shape
+    D = B.shape[1]
+    assert B.shape[0] == H and B.shape[2] == Cdim
+    out = np.empty((Bsz, S, H, D), np.int64)
+    _lib.ora_einsum_bshc_hdc_bshd(_p(A), _p(B), _p(out), rescale, Bsz, S, H, D, Cdim)
+    return out
+
+
+def complex_int64_mul_broadcast(A, B):
+    """A [B,S,H,D,2], B [1,S,1,D,2] (inference/kernel.py:373-395; headDim = A.shape[3])."""
+    A, B = _c(A), _c(B)
+    out = np.empty_like(A)
+    _lib.ora_complex_int64_mul(_p(A), _p(B), _p(out), A.shape[0], A.shape[1], A.shape[2], A.shape[3])
+    return out
+
+
+def rms_stat(A, eps, dim):
+    A = _c(A)
+    M, N = A.shape
+    rms = np.empty((M,), np.int64)
+    rc = _lib.ora_rms_stat(_p(A), _p(rms), M, N, eps, dim)
+    assert rc == 0, "(eps + sum a^2)//dim does not fit 128 bits"
+    return rms
+
+
+def rms_norm_apply(A, W, rms):
+    A, rms = _c(A), _c(rms)
+    M, N = A.shape
+    C = np.empty((M, N), np.int64)
+    if W.dtype == np.int32:
+        W = _c(W, np.int32)
+        _lib.ora_rms_norm_32(_p(A), _p(W), _p(rms), _p(C), M, N)
+    else:
+        W = _c(W)
+        _lib.ora_rms_norm_64(_p(A), _p(W), _p(rms), _p(C), M, N)
+    return C
+
+
+def RMS_Norm_int64(A, W, eps, dim):
+    """(C, rms[:M]) of inference/kernel.py:528-550 (the reference returns its whole 500-row buffer)."""
+    rms = rms_stat(A, eps, dim)
+    return rms_norm_apply(A, W, rms), rms
+
+
+def _lut(fn):
+    lut = np.zeros((256,), np.int64)
+    fn(_p(lut))
+    return lut
+
+
+def softmax_init_q19():
+    return _lut(_lib.ora_softmax_init_q19)
+
+
+def softmax_init_q21():
+    return _lut(_lib.ora_softmax_init_q21)
+
+
+def silu_init_q23():
+    return _lut(_lib.ora_silu_init_q23)
+
+
+def silu_init_q25():
+    return _lut(_lib.ora_silu_init_q25)
+
+
+def _softmax(fn, R, lut):
+    R = _c(R)
+    Bsz, S, H, T = R.shape
+    C = np.empty_like(R)
+    W = np.empty_like(R)
+    fn(_p(R), _p(C), _p(W), _p(_c(lut)), Bsz, S, H, T)
+    return C, W
+
+
+def softmax_q19(R, lut=None):
+    """Returns (C, w): the probabilities and the weights the reference leaves in its input buffer."""
+    return _softmax(_lib.ora_softmax_q19, R, softmax_init_q19() if lut is None else lut)
+
+
+def softmax_q21(R, lut=None):
+    return _softmax(_lib.ora_softmax_q21, R, softmax_init_q21() if lut is None else lut)
+
+
+def _act(fn, R, lut, mode):
+    R = _c(R)
+    C = np.empty_like(R)
+    fn(_p(R), _p(C), _p(_c(lut)), R.size, mode)
+    return C
+
+
+def silu_q23(R, lut=None):
+    return _act(_lib.ora_act_q23, R, silu_init_q23() if lut is None else lut, 0)
+
+
+def sigmoid_q23(R, lut=None):
+    return _act(_lib.ora_act_q23, R, silu_init_q23() if lut is None else lut, 1)
+
+
+def silu_q25(R, lut=None):
+    return _act(_lib.ora_act_q25, R, silu_init_q25() if lut is None else lut, 0)
+
+
+def sigmoid_q25(R, lut=None):
+    return _act(_lib.ora_act_q25, R, silu_init_q25() if lut is None else lut, 1)
