@@ -1,0 +1,131 @@
+/*
+ * int64gemm.h -- C ABI of libint64gemm.so for AMD MI355X (gfx950).
+ *
+ * Drop-in replacement for the shared object that the reference builds from
+ * inference/int64_gemm.cu and loads with ctypes.CDLL("./libint64gemm.so")
+ * (inference/kernel.py:206).  Part 1 declares exactly the entry points that
+ * the reference binds, with the same names, argument order, C types and void
+ * returns.  Part 2 declares additions that have no counterpart in the
+ * reference; nothing in part 1 depends on a caller using them.
+ *
+ * Conventions shared by every entry point (same as the reference):
+ *   - all pointers except the four *_init_* tables are DEVICE pointers owned
+ *     by the caller; tensors are contiguous, row-major, little-endian;
+ *   - work is enqueued on the null (legacy default) stream and the call
+ *     returns without synchronising;
+ *   - no return value.  Unlike the reference, argument and launch errors are
+ *     recorded and can be read with zk_last_error().
+ */
+#ifndef ZK_INT64GEMM_H
+#define ZK_INT64GEMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ======================= Part 1: the reference's ABI ======================= */
+
+/* C[b,m,n] = (sum_k (A[b,m,k]/a_rescale) * (B[n,k]/b_rescale)) >> c_rescale, 128-bit wrapping sum,
+ * `/` truncates toward zero; R = sum mod 2^c_rescale.  A [Bdim,M,K] i64, B [N,K], C,R [Bdim,M,N] i64.
+ * Replaces inference/int64_gemm.cu:79-90 (B int64) and :36-47 (B int32); bound at inference/kernel.py:209-225.
+ * c_rescale must be in [0,63]; the rescales must be non-zero. */
+void int64_64_bmm_broadcast_launcher(const int64_t *A, const int64_t *B, int64_t *C, int64_t *R,
+                                     const int64_t a_rescale, const int64_t b_rescale, const int64_t c_rescale,
+                                     int Bdim, int M, int K, int N);
+void int64_32_bmm_broadcast_launcher(const int64_t *A, const int32_t *B, int64_t *C, int64_t *R,
+                                     const int64_t a_rescale, const int64_t b_rescale, const int64_t c_rescale,
+                                     int Bdim, int M, int K, int N);
+
+/* RoPE: C = A * B as complex numbers in Q42; every real product is bits [42,106) of the 128-bit product.
+ * A,C [batch,seq,heads,headDim,2] i64, B [1,seq,1,headDim,2] i64 (broadcast over batch and heads).
+ * Replaces inference/int64_gemm.cu:274-286; bound at inference/kernel.py:227-232. */
+void complex_int64_mul(const int64_t *A, const int64_t *B, int64_t *C,
+                       int batchSize, int seqLen, int headCount, int headDim);
+
+/* C[s,d] = floor(A[s,d] * W[d] / rms[s]) with a 128-bit product.  A,C [seqLen,Dim] i64, rms [seqLen] i64.
+ * Replaces inference/int64_gemm.cu:365-385; bound at inference/kernel.py:234-248. */
+void rms_norm_32(const int64_t *A, const int32_t *W, const int64_t *rms, int64_t *C, int seqLen, int Dim);
+void rms_norm_64(const int64_t *A, const int64_t *W, const int64_t *rms, int64_t *C, int seqLen, int Dim);
+
+/* MLA einsums, 128-bit accumulation, result (init + sum) >> rescale with init = rescale/2 (half the shift
+ * COUNT) for the first three and 0 for the last.  Replace inference/int64_gemm.cu:416-425, :458-467,
+ * :499-509, :539-549; bound at inference/kernel.py:250-280.
+ *   bshd,hdc->bshc : A [B,S,H,D] i64,  W [H,D,C] i32,   out [B,S,H,C]
+ *   bshc,btc->bsht : A [B,S,H,C] i64,  Bm [B,T,C] i64,  out [B,S,H,T]
+ *   bsht,btc->bshc : A [B,S,H,T] i64,  Bm [B,T,C] i64,  out [B,S,H,C]
+ *   bshc,hdc->bshd : A [B,S,H,C] i64,  W [H,D,C] i32,   out [B,S,H,D]                                   */
+void einsum_bshd_hdc_bshc(const int64_t *q_nope, const int32_t *wkv_b_1, int64_t *out,
+                          int64_t rescale, int B, int S, int H, int D, int C);
+void einsum_bshc_btc_bsht(const int64_t *A, const int64_t *B, int64_t *C,
+                          int64_t rescale, int Bsz, int S, int H, int T, int Cdim);
+void einsum_bsht_btc_bshc(const int64_t *A, const int64_t *B, int64_t *C,
+                          int64_t rescale, int Bsz, int S, int H, int T, int Cdim);
+void einsum_bshc_hdc_bshd(const int64_t *A, const int32_t *B, int64_t *C,
+                          int64_t rescale, int Bsz, int S, int H, int D, int Cdim);
+
+/* Fixed-point softmax over the last dim of R [Bsz,S,H,T] i64 into C; LUT = 256 x i64 on the device.
+ * Replace inference/int64_gemm.cu:661-670 (Q21, rounded divide) and :748-757 (Q19, truncating divide);
+ * bound at inference/kernel.py:282-294.  The reference leaves the per-element weights in R; this
+ * library leaves R untouched unless zk_softmax_clobber_input(1) was called. */
+void softmax_q21(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT, int Bsz, int S, int H, int T);
+void softmax_q19(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT, int Bsz, int S, int H, int T);
+
+/* Fill a HOST table of 256 i64.  Replace inference/int64_gemm.cu:672-680, :759-767, :832-839, :960-967;
+ * bound at inference/kernel.py:296-302, 318-320, 336-338. */
+void softmax_init_q21(int64_t *EXP2_FRAC_LUT);
+void softmax_init_q19(int64_t *EXP2_FRAC_LUT);
+void silu_init_q25(int64_t *EXP2_FRAC_LUT);
+void silu_init_q23(int64_t *EXP2_FRAC_LUT);
+
+/* Elementwise SiLU / sigmoid over R [Bsz,S,Dim] i64 into C.  Replace inference/int64_gemm.cu:821-830,
+ * :884-893, :949-958, :1019-1028; bound at inference/kernel.py:304-334. */
+void silu_q25(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT_25, int Bsz, int S, int Dim);
+void sigmoid_q25(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT_25, int Bsz, int S, int Dim);
+void silu_q23(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT_23, int Bsz, int S, int Dim);
+void sigmoid_q23(int64_t *R, int64_t *C, int64_t *EXP2_FRAC_LUT_23, int Bsz, int S, int Dim);
+
+/* Exported by the reference but bound by none of its Python (inference/int64_gemm.cu:126-132, :173-179,
+ * :215-221): bit-level bf16 / fp32 -> fixed-point conversion of a [rows,cols] matrix. */
+void bf16_to_int32_2d(const uint16_t *input, int32_t *output, int rows, int cols, int rescale);
+void wkv_b_bf16_to_int32(const uint16_t *input, int32_t *output, int rows, int cols);
+void float32_to_int64_2d(const uint32_t *input, int64_t *output, int rows, int cols, int rescale);
+
+/* ================= Part 2: additions (no reference counterpart) ============ */
+
+/* Error channel.  0 = no error since the last zk_clear_error().  Codes: 1 bad argument, 2 launch failure,
+ * 3 unsupported size. */
+int zk_last_error(void);
+const char *zk_last_error_string(void);
+void zk_clear_error(void);
+
+/* RMS statistic on the device: rms[m] = isqrt((eps + sum_n A[m,n]^2) / dim), exact (192-bit sum).
+ * Replaces the host loop of inference/kernel.py:477-494 and :539-542 (one .item() sync per element). */
+void rms_stat_int64(const int64_t *A, int64_t *rms, int M, int N, int64_t eps, int64_t dim);
+
+/* Statistic and normalisation in one launch (the row is read from HBM once); rms [M] is also written. */
+void rms_norm_fused_32(const int64_t *A, const int32_t *W, int64_t *rms, int64_t *C,
+                       int M, int N, int64_t eps, int64_t dim);
+void rms_norm_fused_64(const int64_t *A, const int64_t *W, int64_t *rms, int64_t *C,
+                       int M, int N, int64_t eps, int64_t dim);
+
+/* 1: softmax_q19/q21 also overwrite R with the per-element weights, as the reference's kernels do
+ * (inference/int64_gemm.cu:708,729 and :629,650).  0 (default): R is left untouched. */
+void zk_softmax_clobber_input(int on);
+
+/* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
+ * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
+void zk_gemm_set_path(int path);
+int zk_gemm_get_path(void);
+/* What the last GEMM-like call used: path (1/2) and the limb counts of A and B (0 for the VALU path). */
+void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
+
+/* HIP-event stopwatch on the null stream (the stream every entry point launches on). */
+void zk_timer_start(void);
+float zk_timer_stop_ms(void);   /* records the stop event, waits for it, returns elapsed milliseconds */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZK_INT64GEMM_H */

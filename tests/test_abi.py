@@ -1,0 +1,80 @@
+"""CPU-side checks of the drop-in boundary: the shared object loads, exports every symbol that
+include/int64gemm.h declares, and its host-only table initialisers reproduce the tables the reference's
+circuits hold.  Nothing here launches a kernel."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "zk-deepseek_amd", "libint64gemm.so")
+HEADER = os.path.join(ROOT, "include", "int64gemm.h")
+
+# the 19 symbols whose .argtypes the reference touches at import (inference/kernel.py:209-338):
+# a missing one makes `import kernel` raise AttributeError there
+REFERENCE_BOUND = [
+    "int64_64_bmm_broadcast_launcher", "int64_32_bmm_broadcast_launcher", "complex_int64_mul",
+    "rms_norm_32", "rms_norm_64", "einsum_bshd_hdc_bshc", "einsum_bshc_btc_bsht", "einsum_bsht_btc_bshc",
+    "einsum_bshc_hdc_bshd", "softmax_q21", "softmax_q19", "softmax_init_q21", "softmax_init_q19",
+    "silu_q25", "sigmoid_q25", "silu_init_q25", "silu_q23", "sigmoid_q23", "silu_init_q23",
+]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        import sys
+        sys.path.insert(0, os.path.join(ROOT, "zk-deepseek_amd"))
+        import build
+        build.build(verbose=False)
+    return ctypes.CDLL(LIB)
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?(?:void|int|float|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+
+
+def test_header_declares_reference_abi():
+    names = declared_functions()
+    assert len(names) == len(set(names))
+    for n in REFERENCE_BOUND + ["bf16_to_int32_2d", "wkv_b_bf16_to_int32", "float32_to_int64_2d"]:
+        assert n in names, n
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for n in declared_functions():
+        assert hasattr(lib, n), n
+
+
+def test_table_initialisers_match_reference_tables(lib, zk_tables, oracle):
+    def table(fn):
+        buf = np.zeros(256, np.int64)
+        fn(ctypes.c_void_p(buf.ctypes.data))
+        return buf
+    assert table(lib.softmax_init_q19).tolist() == zk_tables["q19Table"]
+    assert table(lib.silu_init_q23).tolist() == zk_tables["q23Table"]
+    assert np.array_equal(table(lib.softmax_init_q21), oracle.softmax_init_q21())
+    assert np.array_equal(table(lib.silu_init_q25), oracle.silu_init_q25())
+
+
+def test_error_channel_starts_clean(lib):
+    lib.zk_clear_error()
+    assert lib.zk_last_error() == 0
+
+
+def test_kernel_module_mirrors_reference_api():
+    """names model.py imports from kernel (inference/model.py:13-15) plus the wrappers of kernel.py:341-688"""
+    import kernel
+    for n in ["act_quant", "weight_dequant", "fp8_gemm", "int64_bmm_broadcast", "complex_int64_mul_broadcast",
+              "einsum_bshd_hdc_bshc", "einsum_bshc_btc_bsht", "einsum_bsht_btc_bshc", "einsum_bshc_hdc_bshd",
+              "RMS_Norm_int64", "int64_RMS0", "softmax_init_q19", "softmax_init_q21", "silu_init_q23",
+              "silu_init_q25", "softmax_q19", "softmax_q21", "silu_q23", "sigmoid_q23", "silu_q25",
+              "sigmoid_q25", "saveTensor"]:
+        assert callable(getattr(kernel, n)), n
+    assert kernel.rms.shape == (500,) and kernel.rms.device.type == "cpu"
+    with pytest.raises(NotImplementedError):
+        kernel.fp8_gemm()

@@ -1,0 +1,391 @@
+"""Parity of the HIP library against the CPU oracle, bit for bit, through the C ABI (via the `kernel`
+module, whose functions only allocate outputs and pass device pointers).  Needs an MI355X."""
+import numpy as np
+import pytest
+import torch
+
+from util import rand_i32, rand_i64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    import kernel
+    kernel.softmax_init_q19()
+    kernel.softmax_init_q21()
+    kernel.silu_init_q23()
+    kernel.silu_init_q25()
+    kernel.lib.zk_clear_error()
+    yield kernel
+    kernel.lib.zk_gemm_set_path(0)
+    kernel.lib.zk_softmax_clobber_input(0)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+PATHS = [pytest.param(1, id="valu"), pytest.param(2, id="mfma"), pytest.param(0, id="auto")]
+
+
+# ------------------------------------------------------------------------------------ GEMM ------
+def _gemm_case(K, oracle, path, A, W, a_rs, b_rs, c):
+    K.lib.zk_gemm_set_path(path)
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), a_rs, b_rs, c)
+    Ce, Re = oracle.int64_bmm_broadcast(A, W, a_rs, b_rs, c)
+    assert np.array_equal(host(C), Ce), "quotient differs"
+    assert np.array_equal(host(R), Re), "remainder differs"
+
+
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("c", [0, 29])
+def test_gemm_config1_wkv_a(K, oracle, path, c):
+    """BASELINE config 1: Y[16,576] = X[16,7168] @ W[576,7168]^T, X in 2^20, W in 2^16, int64 W."""
+    rng = np.random.default_rng(1000)
+    A = rand_i64(rng, (1, 16, 7168), 20)
+    W = rand_i64(rng, (576, 7168), 16)
+    _gemm_case(K, oracle, path, A, W, 1, 1, c)
+
+
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("bits_a,bits_w,w32,c", [(37, 31, True, 30), (63, 31, True, 29), (63, 63, False, 0),
+                                                 (63, 63, False, 1), (63, 63, False, 29), (63, 63, False, 63),
+                                                 (20, 16, False, 33), (31, 31, False, 16), (47, 40, False, 7)])
+def test_gemm_ranges_and_shifts(K, oracle, path, bits_a, bits_w, w32, c):
+    rng = np.random.default_rng(bits_a * 100 + bits_w + c)
+    A = rand_i64(rng, (2, 70, 300), bits_a)
+    W = rand_i32(rng, (150, 300), bits_w) if w32 else rand_i64(rng, (150, 300), bits_w)
+    if bits_a == 63:
+        A[0, 0, :4] = [-(1 << 63), (1 << 63) - 1, 0x7F7F7F7F7F7F7F80, 0x7F7F7F7F7F7F7F7F]
+    if bits_w == 63:
+        W[0, :4] = [(1 << 63) - 1, -(1 << 63), -0x7F7F7F7F7F7F7F80, 0x7F7F7F7F7F7F7F80]
+    _gemm_case(K, oracle, path, A, W, 1, 1, c)
+
+
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 1, 7, 1), (3, 5, 17, 9), (1, 64, 64, 64), (1, 65, 129, 63),
+                                   (1, 128, 32, 256), (2, 33, 1000, 31), (1, 257, 96, 130)])
+def test_gemm_ragged_shapes(K, oracle, path, shape):
+    Bd, M, Kd, N = shape
+    rng = np.random.default_rng(sum(shape))
+    A = rand_i64(rng, (Bd, M, Kd), 40)
+    W = rand_i64(rng, (N, Kd), 33)
+    _gemm_case(K, oracle, path, A, W, 1, 1, 13)
+
+
+@pytest.mark.parametrize("path", PATHS)
+def test_gemm_operand_divisors(K, oracle, path):
+    """head projection divides the weights by 256 (inference/model.py:1519); division truncates toward zero"""
+    rng = np.random.default_rng(5)
+    A = rand_i64(rng, (1, 9, 200), 45)
+    W = rand_i64(rng, (40, 200), 36)
+    for a_rs, b_rs in ((1, 256), (3, 1), (-7, 5)):
+        _gemm_case(K, oracle, path, A, W, a_rs, b_rs, 21)
+
+
+def test_gemm_rejects_bad_arguments(K):
+    A = torch.zeros((1, 2, 3), dtype=torch.int64, device="cuda")
+    W = torch.zeros((4, 3), dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError):
+        K.int64_bmm_broadcast(A, W, 1, 1, 64)
+    with pytest.raises(RuntimeError):
+        K.int64_bmm_broadcast(A, W, 0, 1, 3)
+    assert K.lib.zk_last_error() == 0          # the wrapper clears the channel after raising
+
+
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("full_range", [False, True])
+def test_gemm_config4_full_size_sampled(K, oracle, path, full_range):
+    """BASELINE config 4 at full size: 512 x 7168 against W[18432,7168].  The oracle checks a sample of rows and
+    columns exactly; linearity in A (at shift 0, where the result is the wrapping int64 product) covers the rest."""
+    if path == 1 and full_range:
+        pytest.skip("one full-size VALU run is enough")
+    g = torch.Generator(device="cpu").manual_seed(4000 + int(full_range))
+    M, Kd, N = 512, 7168, 18432
+    if full_range:
+        A = torch.randint(-(1 << 63), (1 << 63) - 1, (1, M, Kd), generator=g, dtype=torch.int64)
+        W = torch.randint(-(1 << 63), (1 << 63) - 1, (N, Kd), generator=g, dtype=torch.int64)
+    else:
+        A = torch.randint(-(1 << 20), 1 << 20, (1, M, Kd), generator=g, dtype=torch.int64)
+        W = torch.randint(-(1 << 16), 1 << 16, (N, Kd), generator=g, dtype=torch.int64)
+    K.lib.zk_gemm_set_path(path)
+    Ad, Wd = A.cuda(), W.cuda()
+    c = 29
+    C, R = K.int64_bmm_broadcast(Ad, Wd, 1, 1, c)
+    rows = torch.tensor([0, 1, 63, 64, 255, 256, 300, 511])
+    cols = torch.cat([torch.arange(0, 40), torch.arange(9000, 9040), torch.arange(N - 48, N)])
+    Ce, Re = oracle.int64_bmm_broadcast(A[:, rows].numpy(), W[cols].numpy(), 1, 1, c)
+    assert np.array_equal(host(C[:, rows][:, :, cols]), Ce)
+    assert np.array_equal(host(R[:, rows][:, :, cols]), Re)
+    if not full_range:
+        # nothing overflows here: quotient and remainder must rebuild torch's int64 product everywhere
+        full = torch.matmul(A[0, :64], W[:2048].T)          # torch's CPU int64 matmul: the reference's CPU path
+        assert torch.equal((C[0, :64, :2048] * (1 << c) + R[0, :64, :2048]).cpu(), full)
+    # linearity at shift 0: (A1 + A2) W = A1 W + A2 W  (mod 2^64)
+    A2 = torch.roll(Ad, 1, dims=1)
+    C0, _ = K.int64_bmm_broadcast(Ad, Wd, 1, 1, 0)
+    C1, _ = K.int64_bmm_broadcast(A2, Wd, 1, 1, 0)
+    C2, _ = K.int64_bmm_broadcast(Ad + A2, Wd, 1, 1, 0)
+    assert torch.equal(C2, C0 + C1)
+    assert torch.equal(C1, torch.roll(C0, 1, dims=1))
+
+
+# ---------------------------------------------------------------------------------- einsums -----
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("bits", [20, 40, 63])
+def test_einsums(K, oracle, path, bits):
+    K.lib.zk_gemm_set_path(path)
+    rng = np.random.default_rng(bits)
+    B, S, H, D, Cc, T = 2, 9, 5, 24, 40, 70
+    q = rand_i64(rng, (B, S, H, D), bits)
+    w1 = rand_i32(rng, (H, D, Cc))
+    a = rand_i64(rng, (B, S, H, Cc), bits)
+    kv = rand_i64(rng, (B, T, Cc), bits)
+    p = rand_i64(rng, (B, S, H, T), bits)
+    w2 = rand_i32(rng, (H, D, Cc))
+    for rescale in (0, 21, 23, 37):
+        assert np.array_equal(host(K.einsum_bshd_hdc_bshc(dev(q), dev(w1), rescale)),
+                              oracle.einsum_bshd_hdc_bshc(q, w1, rescale))
+        assert np.array_equal(host(K.einsum_bshc_btc_bsht(dev(a), dev(kv), rescale)),
+                              oracle.einsum_bshc_btc_bsht(a, kv, rescale))
+        assert np.array_equal(host(K.einsum_bsht_btc_bshc(dev(p), dev(kv), rescale)),
+                              oracle.einsum_bsht_btc_bshc(p, kv, rescale))
+        assert np.array_equal(host(K.einsum_bshc_hdc_bshd(dev(a), dev(w2), rescale)),
+                              oracle.einsum_bshc_hdc_bshd(a, w2, rescale))
+
+
+@pytest.mark.parametrize("path", PATHS)
+def test_einsums_model_shapes(K, oracle, path):
+    """MLA absorb shapes at a short prefill: H=128, nope 128, kv_lora 512, rope 64 (inference/model.py:862-951)."""
+    K.lib.zk_gemm_set_path(path)
+    rng = np.random.default_rng(77)
+    B, S, H, T = 1, 4, 128, 12
+    q_nope = rand_i64(rng, (B, S, H, 128), 24)
+    wkv_b_1 = rand_i32(rng, (H, 128, 512), 28)
+    qn = K.einsum_bshd_hdc_bshc(dev(q_nope), dev(wkv_b_1), 33)
+    assert np.array_equal(host(qn), oracle.einsum_bshd_hdc_bshc(q_nope, wkv_b_1, 33))
+    kvc = rand_i64(rng, (B, T, 512), 26)
+    s1 = K.einsum_bshc_btc_bsht(qn, dev(kvc), 23)
+    assert np.array_equal(host(s1), oracle.einsum_bshc_btc_bsht(host(qn), kvc, 23))
+    q_pe = rand_i64(rng, (B, S, H, 64), 22)
+    pec = rand_i64(rng, (B, T, 64), 24)
+    s2 = K.einsum_bshc_btc_bsht(dev(q_pe), dev(pec), 21)
+    assert np.array_equal(host(s2), oracle.einsum_bshc_btc_bsht(q_pe, pec, 21))
+    P = rand_i64(rng, (B, S, H, T), 19)
+    o = K.einsum_bsht_btc_bshc(dev(P), dev(kvc), 23)
+    assert np.array_equal(host(o), oracle.einsum_bsht_btc_bshc(P, kvc, 23))
+    wkv_b_2 = rand_i32(rng, (H, 128, 512), 28)
+    x = K.einsum_bshc_hdc_bshd(o, dev(wkv_b_2), 31)
+    assert np.array_equal(host(x), oracle.einsum_bshc_hdc_bshd(host(o), wkv_b_2, 31))
+
+
+# ---------------------------------------------------------------------------------- softmax -----
+def _scores(rng, shape, Q, masked=True):
+    x = rng.integers(-(12 << Q), 12 << Q, size=shape, dtype=np.int64)
+    if masked and shape[-1] > 1:
+        T = shape[-1]
+        cut = rng.integers(1, T + 1, size=shape[:-1])
+        x = np.where(np.arange(T) < cut[..., None], x, x - (1 << 42))       # causal-mask value -(64 << 36)
+    return x
+
+
+@pytest.mark.parametrize("fn,Q", [("softmax_q19", 19), ("softmax_q21", 21)])
+@pytest.mark.parametrize("T", [1, 2, 3, 7, 64, 100, 127, 128, 129, 256, 257, 1000, 1024, 1025, 2048, 2049, 5000])
+def test_softmax_lengths(K, oracle, fn, Q, T):
+    rng = np.random.default_rng(T + Q)
+    x = _scores(rng, (1, 3, 5, T), Q)
+    R = dev(x)
+    C = torch.empty_like(R)
+    getattr(K, fn)(R, C)
+    Ce, _ = getattr(oracle, fn)(x)
+    assert np.array_equal(host(C), Ce)
+    assert np.array_equal(host(R), x), "input must stay intact by default"
+
+
+@pytest.mark.parametrize("fn", ["softmax_q19", "softmax_q21"])
+@pytest.mark.parametrize("T", [96, 1024, 3001])
+def test_softmax_reference_clobber_mode(K, oracle, fn, T):
+    """with the switch on, the input buffer ends up holding the weights, as after the reference's kernel"""
+    rng = np.random.default_rng(T)
+    x = _scores(rng, (2, 2, 4, T), 19)
+    R = dev(x)
+    C = torch.empty_like(R)
+    K.lib.zk_softmax_clobber_input(1)
+    try:
+        getattr(K, fn)(R, C)
+    finally:
+        K.lib.zk_softmax_clobber_input(0)
+    Ce, We = getattr(oracle, fn)(x)
+    assert np.array_equal(host(C), Ce)
+    assert np.array_equal(host(R), We)
+
+
+@pytest.mark.parametrize("fn", ["softmax_q19", "softmax_q21"])
+def test_softmax_hostile_inputs(K, oracle, fn):
+    """full-range scores and an arbitrary table: the slow exact paths must agree with the oracle's fixed semantics"""
+    rng = np.random.default_rng(9)
+    x = rand_i64(rng, (1, 2, 6, 333), 63)
+    x[0, 0, 0, :] = 7
+    x[0, 0, 1, :] = -(1 << 63)
+    lut = rand_i64(rng, (256,), 63)
+    for table in (None, lut):
+        R = dev(x)
+        C = torch.empty_like(R)
+        t = dev(table) if table is not None else (K.EXP2_FRAC_LUT_Q19 if fn == "softmax_q19" else K.EXP2_FRAC_LUT_Q21)
+        getattr(K.lib, fn)(R.data_ptr(), C.data_ptr(), t.data_ptr(), 1, 2, 6, 333)
+        torch.cuda.synchronize()
+        Ce, _ = getattr(oracle, fn)(x, table)
+        assert np.array_equal(host(C), Ce)
+
+
+def test_softmax_unaligned_rows(K, oracle):
+    rng = np.random.default_rng(3)
+    x = _scores(rng, (1, 2, 3, 1024), 19)
+    buf = torch.zeros(x.size + 1, dtype=torch.int64, device="cuda")
+    R = buf[1:].view(1, 2, 3, 1024)                 # 8-byte aligned only
+    R.copy_(dev(x))
+    C = torch.empty_like(dev(x))
+    K.softmax_q19(R, C)
+    assert np.array_equal(host(C), oracle.softmax_q19(x)[0])
+
+
+def test_softmax_config3_full_size_properties(K, oracle):
+    """BASELINE config 3 softmax at full size [1,1024,128,1024]: exact on a sample of rows, invariants on all."""
+    g = torch.Generator(device="cpu").manual_seed(3000)
+    S, H, T = 1024, 128, 1024
+    x = torch.randint(-(6 << 19), 6 << 19, (1, S, H, T), generator=g, dtype=torch.int64)
+    mask = torch.full((S, T), -(64 << 36), dtype=torch.int64).triu_(1)
+    x += mask.unsqueeze(1)
+    R = x.cuda()
+    C = torch.empty_like(R)
+    K.softmax_q19(R, C)
+    assert torch.equal(R.cpu(), x)
+    sel = [0, 1, 17, 511, 1023]
+    Ce, _ = oracle.softmax_q19(x[:, sel].numpy())
+    assert np.array_equal(host(C[:, sel]), Ce)
+    assert int(C.min()) >= 0 and int(C.max()) <= 1 << 19
+    sums = C.sum(-1)
+    assert int(sums.max()) <= 1 << 19 and int(sums.min()) > (1 << 19) - T
+    causal = torch.ones((S, T), dtype=torch.bool, device="cuda").triu_(1)
+    assert int((C * causal.unsqueeze(1)).abs().max()) == 0            # masked positions get exactly 0
+
+
+# -------------------------------------------------------------------------------- SiLU / sigmoid --
+ACTS = [("silu_q23", 23), ("sigmoid_q23", 23), ("silu_q25", 25), ("sigmoid_q25", 25)]
+
+
+@pytest.mark.parametrize("fn,Q", ACTS)
+@pytest.mark.parametrize("shape", [(1, 1, 1), (1, 3, 7), (2, 5, 256), (1, 128, 2048), (1, 7, 2049)])
+def test_activation_shapes(K, oracle, fn, Q, shape):
+    rng = np.random.default_rng(Q + sum(shape))
+    x = rng.integers(-(20 << Q), 20 << Q, size=shape, dtype=np.int64)
+    R = dev(x)
+    C = torch.empty_like(R)
+    getattr(K, fn)(R, C)
+    assert np.array_equal(host(C), getattr(oracle, fn)(x))
+    assert np.array_equal(host(R), x)
+
+
+@pytest.mark.parametrize("fn,Q", ACTS)
+def test_activation_edges_and_hazard_region(K, oracle, fn, Q):
+    """saturation limits, zero, the overflowing-shift region x <= -27.7 (k >= 40), full-range garbage and a
+    hostile table: everything must match the oracle's fixed semantics bit for bit"""
+    one = 1 << Q
+    rng = np.random.default_rng(Q)
+    edges = np.array([0, 1, -1, 64 * one, 64 * one - 1, -64 * one, -64 * one + 1, 100 * one, -100 * one,
+                      -(1 << 63), (1 << 63) - 1, -28 * one, -44 * one, -45 * one, -63 * one], np.int64)
+    x = np.concatenate([edges, rng.integers(-64 * one, -27 * one, size=3000, dtype=np.int64),
+                        rand_i64(rng, (3000,), 63)]).reshape(1, 1, -1)
+    lut_bad = rand_i64(rng, (256,), 63)
+    default = K.EXP2_FRAC_LUT_Q23 if Q == 23 else K.EXP2_FRAC_LUT_Q25
+    for table in (None, lut_bad):
+        R = dev(x)
+        C = torch.empty_like(R)
+        t = default if table is None else dev(table)
+        getattr(K.lib, fn)(R.data_ptr(), C.data_ptr(), t.data_ptr(), 1, 1, x.shape[2])
+        torch.cuda.synchronize()
+        assert np.array_equal(host(C), getattr(oracle, fn)(x, table))
+
+
+def test_activation_unaligned_pointers(K, oracle):
+    rng = np.random.default_rng(8)
+    x = rng.integers(-(20 << 23), 20 << 23, size=(1, 3, 1001), dtype=np.int64)
+    buf = torch.zeros(x.size + 1, dtype=torch.int64, device="cuda")
+    R = buf[1:].view(1, 3, 1001)
+    R.copy_(dev(x))
+    C = torch.empty_like(dev(x))
+    K.silu_q23(R, C)
+    assert np.array_equal(host(C), oracle.silu_q23(x))
+
+
+def test_activation_dense_ffn_shape(K, oracle):
+    """[1,512,18432], the dense-FFN activation shape; oracle on everything (9.4 M elements)."""
+    g = torch.Generator(device="cpu").manual_seed(2300)
+    x = torch.randint(-(16 << 23), 16 << 23, (1, 512, 18432), generator=g, dtype=torch.int64)
+    R = x.cuda()
+    C = torch.empty_like(R)
+    oracle.set_threads(oracle.max_threads())
+    for fn in ("silu_q23", "sigmoid_q23"):
+        getattr(K, fn)(R, C)
+        assert np.array_equal(host(C), getattr(oracle, fn)(x.numpy()))
+    oracle.set_threads(1)
+
+
+# ---------------------------------------------------------------------------------- RMSNorm -----
+@pytest.mark.parametrize("bits", [20, 37, 63])
+@pytest.mark.parametrize("N", [7, 512, 1536, 7168, 9001])
+@pytest.mark.parametrize("w32", [True, False])
+def test_rmsnorm(K, oracle, bits, N, w32):
+    rng = np.random.default_rng(bits + N)
+    M = 6
+    A = rand_i64(rng, (M, N), bits)
+    if bits == 63:
+        A[0, :] = (1 << 63) - 1
+    W = rng.integers(1 << 5, 1 << 20, size=(N,), dtype=np.int32) if w32 else rand_i64(rng, (N,), 40)
+    C, rms = K.RMS_Norm_int64(dev(A), dev(W), 1, N)
+    Ce, rmse = oracle.RMS_Norm_int64(A, W, 1, N)
+    assert rms.shape == (500,) and rms.device.type == "cpu"
+    assert np.array_equal(rms[:M].numpy(), rmse)
+    assert np.array_equal(host(C), Ce)
+
+
+def test_rmsnorm_reference_entry_points(K, oracle):
+    """rms_norm_32 / rms_norm_64 with a caller-supplied rms vector (the reference's contract), including
+    negative and huge divisors that only the slow exact path handles"""
+    rng = np.random.default_rng(12)
+    A = rand_i64(rng, (5, 300), 63)
+    rms = np.array([1, -3, 12345678901, (1 << 62) + 12345, 977], np.int64)
+    for W in (rand_i32(rng, (300,)), rand_i64(rng, (300,), 63)):
+        C = torch.empty((5, 300), dtype=torch.int64, device="cuda")
+        fn = K.lib.rms_norm_32 if W.dtype == np.int32 else K.lib.rms_norm_64
+        Ad, Wd, rd = dev(A), dev(W), dev(rms)
+        fn(Ad.data_ptr(), Wd.data_ptr(), rd.data_ptr(), C.data_ptr(), 5, 300)
+        torch.cuda.synchronize()
+        assert np.array_equal(host(C), oracle.rms_norm_apply(A, W, rms))
+    assert K.int64_RMS0(dev(A[0]), 1, 300) == int(oracle.rms_stat(A[:1], 1, 300)[0])
+
+
+def test_rmsnorm_model_shape(K, oracle):
+    """[256,7168] at residual-stream magnitudes (|x| up to ~2^37, Q31) with int32 Q21 weights"""
+    g = torch.Generator(device="cpu").manual_seed(600)
+    A = torch.randint(-(1 << 37), 1 << 37, (256, 7168), generator=g, dtype=torch.int64)
+    W = torch.randint(1 << 18, 1 << 20, (7168,), generator=g, dtype=torch.int32)
+    C, rms = K.RMS_Norm_int64(A.cuda(), W.cuda(), 1, 7168)
+    Ce, rmse = oracle.RMS_Norm_int64(A.numpy(), W.numpy(), 1, 7168)
+    assert np.array_equal(rms[:256].numpy(), rmse) and np.array_equal(host(C), Ce)
+
+
+# ------------------------------------------------------------------------------------- RoPE -----
+@pytest.mark.parametrize("bits", [31, 63])
+def test_rope(K, oracle, bits):
+    rng = np.random.default_rng(bits)
+    A = rand_i64(rng, (2, 7, 5, 32, 2), bits)
+    Bt = rand_i64(rng, (1, 7, 1, 32, 2), 43)
+    out = K.complex_int64_mul_broadcast(dev(A), dev(Bt))
+    assert np.array_equal(host(out), oracle.complex_int64_mul_broadcast(A, Bt))

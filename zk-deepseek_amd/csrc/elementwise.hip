@@ -1,0 +1,249 @@
+// Elementwise int64 fixed-point kernels: SiLU / sigmoid (Q23, Q25), the RoPE complex multiply and the
+// three float -> fixed-point converters.  All are HBM-bound: 16-byte loads and stores, one pass.
+#include "common.h"
+#include "../../include/int64gemm.h"
+
+namespace zk {
+
+struct __attribute__((aligned(16))) i64x2 { int64_t x, y; };
+
+// -------------------------------------------------------------------------------------------------
+// SiLU / sigmoid.  sigma(x) = 1 / (1 + e^-x) with e^-x = 2^y, y = -x*log2(e) split into an integer part
+// k (a shift) and a fraction looked up in a 256-entry table; the reciprocal is an exact integer divide.
+// Follows inference/int64_gemm.cu:903-947, :969-1017 (Q23) and :775-819, :841-882 (Q25).
+// -------------------------------------------------------------------------------------------------
+template <int Q> struct ActConst;
+template <> struct ActConst<23> { static constexpr int64_t kLog2e = 12102203; };
+template <> struct ActConst<25> { static constexpr int64_t kLog2e = 48408813; };
+
+template <int Q, bool SIGMOID>
+__device__ __forceinline__ int64_t act_one(int64_t r, const int64_t *lut)
+{
+    constexpr int64_t LIM = (int64_t)64 << Q;
+    constexpr int64_t ONE = (int64_t)1 << Q;
+    if (r >= LIM) return r;     // the sigmoid kernels return x here as well
+    if (r <= -LIM) return 0;
+    // |r| < 2^(Q+6) and log2(e)*2^Q < 2^(Q+1): the product needs 2Q+8 <= 58 bits, so int64 is exact.
+    int64_t y;
+    if (Q == 23) y = ((-r) * ActConst<Q>::kLog2e) >> Q;    // negate, multiply, shift
+    else y = -((r * ActConst<Q>::kLog2e) >> Q);             // multiply, shift, negate
+    int64_t k = y >> Q;
+    int64_t f = y & (ONE - 1);
+    int64_t t = lut[f >> (Q - 8)];
+    int64_t u = 0;
+    if (k > -63) {
+        if (k < 0) u = t >> (int)(-k);
+        else u = (k >= 64) ? 0 : (int64_t)((uint64_t)t << (int)k);    // shifts of 64 or more give 0
+    }
+    int64_t den = (int64_t)((uint64_t)ONE + (uint64_t)u);
+    int64_t q;
+    if (den >= ONE && den < ((int64_t)1 << 53)) {
+        constexpr uint64_t NUM = (uint64_t)1 << (2 * Q);
+        q = (int64_t)udiv_by_inv(NUM, (uint64_t)den, 1.0 / (double)den);
+    } else {
+        q = tdiv64((int64_t)1 << (2 * Q), den);
+    }
+    if (SIGMOID) return q;
+    return (int64_t)((uint64_t)r * (uint64_t)q) >> Q;
+}
+
+constexpr int kActThreads = 256;
+constexpr int kActUnroll = 4;
+
+template <int Q, bool SIGMOID, bool VEC>
+__global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restrict__ R, int64_t *__restrict__ C,
+                                                          const int64_t *__restrict__ lut_g, long n)
+{
+    __shared__ int64_t lut[256];
+    lut[threadIdx.x] = lut_g[threadIdx.x];
+    __syncthreads();
+    if (VEC) {
+        long nvec = n >> 1;
+        long base = (long)blockIdx.x * (kActThreads * kActUnroll) + threadIdx.x;
+        i64x2 v[kActUnroll];
+#pragma unroll
+        for (int j = 0; j < kActUnroll; j++) {
+            long i = base + (long)j * kActThreads;
+            if (i < nvec) v[j] = reinterpret_cast<const i64x2 *>(R)[i];
+        }
+#pragma unroll
+        for (int j = 0; j < kActUnroll; j++) {
+            long i = base + (long)j * kActThreads;
+            if (i < nvec) {
+                i64x2 o;
+                o.x = act_one<Q, SIGMOID>(v[j].x, lut);
+                o.y = act_one<Q, SIGMOID>(v[j].y, lut);
+                reinterpret_cast<i64x2 *>(C)[i] = o;
+            }
+        }
+        if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) C[n - 1] = act_one<Q, SIGMOID>(R[n - 1], lut);
+    } else {
+        long base = (long)blockIdx.x * (kActThreads * kActUnroll) + threadIdx.x;
+#pragma unroll
+        for (int j = 0; j < kActUnroll; j++) {
+            long i = base + (long)j * kActThreads;
+            if (i < n) C[i] = act_one<Q, SIGMOID>(R[i], lut);
+        }
+    }
+}
+
+template <int Q, bool SIGMOID>
+static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim)
+{
+    if (Bsz < 0 || S < 0 || Dim < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
+    long n = (long)Bsz * S * Dim;
+    if (n == 0) return;
+    if (!R || !C || !lut) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    bool vec = (((uintptr_t)R | (uintptr_t)C) & 15) == 0;
+    long per_block = (long)kActThreads * kActUnroll;
+    long items = vec ? ((n >> 1) > 0 ? (n >> 1) : 1) : n;
+    long blocks = (items + per_block - 1) / per_block;
+    if (vec) act_kernel<Q, SIGMOID, true><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n);
+    else act_kernel<Q, SIGMOID, false><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n);
+    check_launch(name);
+}
+
+// -------------------------------------------------------------------------------------------------
+// RoPE: (a0 + i a1) * (b0 + i b1) in Q42.  Each real product keeps bits [42,106) of the signed 128-bit
+// product (inference/int64_gemm.cu:257-263); the table is broadcast over batch and heads (:245).
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int64_t mul_q42(int64_t a, int64_t b)
+{
+    uint64_t lo = (uint64_t)a * (uint64_t)b;
+    uint64_t hi = (uint64_t)__mul64hi((long long)a, (long long)b);
+    return (int64_t)((hi << 22) | (lo >> 42));
+}
+
+__global__ __launch_bounds__(256) void rope_kernel(const i64x2 *__restrict__ A, const i64x2 *__restrict__ Bt,
+                                                   i64x2 *__restrict__ C, long total, int seq, int heads, int headDim)
+{
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    long i = idx;
+    int d = (int)(i % headDim);
+    i /= headDim;
+    i /= heads;
+    int s = (int)(i % seq);
+    i64x2 a = A[idx];
+    i64x2 b = Bt[(long)s * headDim + d];
+    i64x2 o;
+    o.x = (int64_t)((uint64_t)mul_q42(a.x, b.x) - (uint64_t)mul_q42(a.y, b.y));
+    o.y = (int64_t)((uint64_t)mul_q42(a.x, b.y) + (uint64_t)mul_q42(a.y, b.x));
+    C[idx] = o;
+}
+
+// -------------------------------------------------------------------------------------------------
+// float bit patterns -> fixed point (inference/int64_gemm.cu:92-221).  value = (1.mantissa) * 2^(exp+rescale)
+// truncated toward zero; shifts the reference leaves to the hardware are fixed as: left shift of 32 or more
+// gives 0, right shift of 32 or more gives 0.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t scale_mantissa_u32(uint32_t r2, int ex2)
+{
+    if (ex2 >= 0) return ex2 >= 32 ? 0u : r2 * (1u << ex2);
+    return -ex2 >= 31 ? 0u : r2 / (1u << -ex2);
+}
+
+__global__ __launch_bounds__(256) void bf16_to_int32_kernel(const uint16_t *__restrict__ in, int32_t *__restrict__ out,
+                                                            long n, int rescale, int wkv_b)
+{
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    int v0 = in[idx];
+    int ex0 = ((v0 >> 7) & 0xFF) - 127;
+    int r0 = v0 & 0x7F;
+    if (ex0 == -127 && r0 == 0) { out[idx] = 0; return; }
+    if (wkv_b && ex0 >= -1) { out[idx] = 0x7FFFFFFF; return; }       // saturate |x| >= 0.5 (:151-154)
+    uint32_t v = scale_mantissa_u32((uint32_t)(r0 + 128), ex0 + rescale);
+    if (v0 & 0x8000) v = 0u - v;
+    out[idx] = (int32_t)v;
+}
+
+__global__ __launch_bounds__(256) void f32_to_int64_kernel(const uint32_t *__restrict__ in, int64_t *__restrict__ out,
+                                                           long n, int rescale)
+{
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    uint32_t v0 = in[idx];
+    int ex0 = (int)((v0 >> 23) & 0xFF) - 127;
+    int r0 = (int)(v0 & 0x7FFFFF);
+    if (ex0 == -127 && r0 == 0) { out[idx] = 0; return; }
+    int ex2 = ex0 + rescale;
+    int64_t r2 = (int64_t)r0 + 8388608;
+    int64_t v;
+    // the reference multiplies by a 32-bit `1 << ex2` (:202): the factor wraps to INT_MIN at 31 and is 0 beyond
+    if (ex2 >= 0) v = ex2 >= 32 ? 0 : (int64_t)((uint64_t)r2 * (uint64_t)(int64_t)(int32_t)(1u << ex2));
+    else v = -ex2 >= 31 ? 0 : r2 / (int64_t)(1u << -ex2);
+    if (v0 & 0x80000000u) v = (int64_t)(0 - (uint64_t)v);
+    out[idx] = v;
+}
+
+}  // namespace zk
+
+extern "C" {
+
+void silu_q23(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
+{
+    zk::launch_act<23, false>("silu_q23", R, C, lut, Bsz, S, Dim);
+}
+void sigmoid_q23(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
+{
+    zk::launch_act<23, true>("sigmoid_q23", R, C, lut, Bsz, S, Dim);
+}
+void silu_q25(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
+{
+    zk::launch_act<25, false>("silu_q25", R, C, lut, Bsz, S, Dim);
+}
+void sigmoid_q25(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
+{
+    zk::launch_act<25, true>("sigmoid_q25", R, C, lut, Bsz, S, Dim);
+}
+
+void complex_int64_mul(const int64_t *A, const int64_t *B, int64_t *C, int batchSize, int seqLen, int headCount,
+                       int headDim)
+{
+    if (batchSize < 0 || seqLen < 0 || headCount < 0 || headDim < 0) {
+        zk::set_error(zk::kBadArgument, "complex_int64_mul: negative dimension");
+        return;
+    }
+    long total = (long)batchSize * seqLen * headCount * headDim;
+    if (total == 0) return;
+    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "complex_int64_mul: null pointer"); return; }
+    if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) {
+        zk::set_error(zk::kBadArgument, "complex_int64_mul: pointers must be 16-byte aligned");
+        return;
+    }
+    long blocks = (total + 255) / 256;
+    zk::rope_kernel<<<dim3((unsigned)blocks), dim3(256), 0, 0>>>(
+        reinterpret_cast<const zk::i64x2 *>(A), reinterpret_cast<const zk::i64x2 *>(B),
+        reinterpret_cast<zk::i64x2 *>(C), total, seqLen, headCount, headDim);
+    zk::check_launch("complex_int64_mul");
+}
+
+void bf16_to_int32_2d(const uint16_t *input, int32_t *output, int rows, int cols, int rescale)
+{
+    long n = (long)rows * cols;
+    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "bf16_to_int32_2d: negative dimension"); return; }
+    if (n == 0) return;
+    zk::bf16_to_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, rescale, 0);
+    zk::check_launch("bf16_to_int32_2d");
+}
+
+void wkv_b_bf16_to_int32(const uint16_t *input, int32_t *output, int rows, int cols)
+{
+    long n = (long)rows * cols;
+    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "wkv_b_bf16_to_int32: negative dimension"); return; }
+    if (n == 0) return;
+    zk::bf16_to_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, 25, 1);
+    zk::check_launch("wkv_b_bf16_to_int32");
+}
+
+void float32_to_int64_2d(const uint32_t *input, int64_t *output, int rows, int cols, int rescale)
+{
+    long n = (long)rows * cols;
+    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "float32_to_int64_2d: negative dimension"); return; }
+    if (n == 0) return;
+    zk::f32_to_int64_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, rescale);
+    zk::check_launch("float32_to_int64_2d");
+}
+
+}  // extern "C"

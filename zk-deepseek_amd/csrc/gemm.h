@@ -1,0 +1,39 @@
+// One descriptor for every GEMM-shaped entry point (the two bmm launchers and the four MLA einsums):
+//
+//   C[g][m][n] = (init + sum_k (A[g][m][k] / a_rs) * (B[g][n,k] / b_rs)) >> shift      (128-bit wrapping sum)
+//   R[g][m][n] = (that sum) mod 2^shift                                                 (optional)
+//
+// A is always k-contiguous.  B is either k-contiguous ("n-major", ldbk == 1: weights [N,K], K^T of the
+// attention scores) or n-contiguous ("k-major", ldbn == 1: V of P.V, wkv_b_1 [D,C]).
+#pragma once
+#include "common.h"
+
+namespace zk {
+
+struct GemmDesc {
+    const int64_t *A;
+    long lda, sA;             // A[g][m][k] = A[g * sA + m * lda + k]
+    const void *B;
+    int b32;                  // 1: B holds int32, 0: int64
+    long ldbn, ldbk, sB;      // B[g][n,k] = B[g * sB + n * ldbn + k * ldbk]; exactly one of ldbn, ldbk is 1
+    int64_t *C, *R;           // R may be null
+    long ldc, sC;             // C[g][m][n] = C[g * sC + m * ldc + n]
+    int G, M, N, K;
+    int shift;                // 0..63
+    int64_t init;             // added to the sum before the shift
+    int64_t a_rs, b_rs;       // operand divisors (truncating), 1 = none
+};
+
+enum GemmPath { kPathAuto = 0, kPathValu = 1, kPathMfma = 2 };
+
+// Native 64-bit multiply-add chains on the vector ALU; handles every descriptor.
+void gemm_valu_launch(const GemmDesc &d);
+
+// Limb-decomposed i8 MFMA.  Returns false (nothing launched) when the descriptor is outside what it
+// supports, in which case the caller falls back to the VALU path.
+bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
+
+// Top-level dispatch used by the extern "C" launchers.
+void gemm_dispatch(const char *name, const GemmDesc &d);
+
+}  // namespace zk

@@ -1,0 +1,155 @@
+// extern "C" launchers of the GEMM-shaped entry points: argument checks, descriptor construction and the
+// choice between the VALU and the MFMA instruction path.
+#include "gemm.h"
+#include "../../include/int64gemm.h"
+
+namespace zk {
+
+static int g_gemm_path = kPathAuto;
+static int g_last_path = 0, g_last_la = 0, g_last_lb = 0;
+
+void gemm_dispatch(const char *name, const GemmDesc &d)
+{
+    if (g_gemm_path != kPathValu) {
+        int la = 0, lb = 0;
+        if (gemm_mfma_launch(d, &la, &lb)) {
+            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb;
+            check_launch(name);
+            return;
+        }
+        if (zk_last_error() != kOk) return;
+    }
+    gemm_valu_launch(d);
+    g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+    check_launch(name);
+}
+
+static bool dims_ok(const char *name, std::initializer_list<int> dims, int64_t shift)
+{
+    for (int v : dims)
+        if (v < 0) { set_error(kBadArgument, "%s: negative dimension", name); return false; }
+    if (shift < 0 || shift > 63) {
+        set_error(kBadArgument, "%s: shift %lld outside [0,63]", name, (long long)shift);
+        return false;
+    }
+    return true;
+}
+
+static void bmm(const char *name, const int64_t *A, const void *B, int b32, int64_t *C, int64_t *R,
+                int64_t a_rs, int64_t b_rs, int64_t c_rs, int Bdim, int M, int K, int N)
+{
+    if (!dims_ok(name, { Bdim, M, K, N }, c_rs)) return;
+    if (a_rs == 0 || b_rs == 0) { set_error(kBadArgument, "%s: zero rescale divisor", name); return; }
+    if ((long)Bdim * M * N == 0) return;
+    if (!A || !B || !C) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    GemmDesc d;
+    d.A = A; d.lda = K; d.sA = (long)M * K;
+    d.B = B; d.b32 = b32; d.ldbn = K; d.ldbk = 1; d.sB = 0;
+    d.C = C; d.R = R; d.ldc = N; d.sC = (long)M * N;
+    d.G = Bdim; d.M = M; d.N = N; d.K = K;
+    d.shift = (int)c_rs; d.init = 0; d.a_rs = a_rs; d.b_rs = b_rs;
+    gemm_dispatch(name, d);
+}
+
+}  // namespace zk
+
+extern "C" {
+
+void int64_64_bmm_broadcast_launcher(const int64_t *A, const int64_t *B, int64_t *C, int64_t *R,
+                                     const int64_t a_rescale, const int64_t b_rescale, const int64_t c_rescale,
+                                     int Bdim, int M, int K, int N)
+{
+    zk::bmm("int64_64_bmm_broadcast_launcher", A, B, 0, C, R, a_rescale, b_rescale, c_rescale, Bdim, M, K, N);
+}
+
+void int64_32_bmm_broadcast_launcher(const int64_t *A, const int32_t *B, int64_t *C, int64_t *R,
+                                     const int64_t a_rescale, const int64_t b_rescale, const int64_t c_rescale,
+                                     int Bdim, int M, int K, int N)
+{
+    zk::bmm("int64_32_bmm_broadcast_launcher", A, B, 1, C, R, a_rescale, b_rescale, c_rescale, Bdim, M, K, N);
+}
+
+// out[b,s,h,c] = (rescale/2 + sum_d q[b,s,h,d] * W[h,d,c]) >> rescale: one GEMM per head, rows (b,s).
+void einsum_bshd_hdc_bshc(const int64_t *q_nope, const int32_t *wkv_b_1, int64_t *out, int64_t rescale,
+                          int B, int S, int H, int D, int C)
+{
+    const char *name = "einsum_bshd_hdc_bshc";
+    if (!zk::dims_ok(name, { B, S, H, D, C }, rescale)) return;
+    if ((long)B * S * H * C == 0) return;
+    if (!q_nope || !wkv_b_1 || !out) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    zk::GemmDesc d;
+    d.A = q_nope; d.lda = (long)H * D; d.sA = D;
+    d.B = wkv_b_1; d.b32 = 1; d.ldbn = 1; d.ldbk = C; d.sB = (long)D * C;
+    d.C = out; d.R = nullptr; d.ldc = (long)H * C; d.sC = C;
+    d.G = H; d.M = B * S; d.N = C; d.K = D;
+    d.shift = (int)rescale; d.init = rescale / 2; d.a_rs = 1; d.b_rs = 1;
+    zk::gemm_dispatch(name, d);
+}
+
+// out[b,s,h,t] = (rescale/2 + sum_c A[b,s,h,c] * Bm[b,t,c]) >> rescale: one GEMM per batch, rows (s,h).
+void einsum_bshc_btc_bsht(const int64_t *A, const int64_t *B, int64_t *C, int64_t rescale,
+                          int Bsz, int S, int H, int T, int Cdim)
+{
+    const char *name = "einsum_bshc_btc_bsht";
+    if (!zk::dims_ok(name, { Bsz, S, H, T, Cdim }, rescale)) return;
+    if ((long)Bsz * S * H * T == 0) return;
+    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    zk::GemmDesc d;
+    d.A = A; d.lda = Cdim; d.sA = (long)S * H * Cdim;
+    d.B = B; d.b32 = 0; d.ldbn = Cdim; d.ldbk = 1; d.sB = (long)T * Cdim;
+    d.C = C; d.R = nullptr; d.ldc = T; d.sC = (long)S * H * T;
+    d.G = Bsz; d.M = S * H; d.N = T; d.K = Cdim;
+    d.shift = (int)rescale; d.init = rescale / 2; d.a_rs = 1; d.b_rs = 1;
+    zk::gemm_dispatch(name, d);
+}
+
+// out[b,s,h,c] = (rescale/2 + sum_t P[b,s,h,t] * V[b,t,c]) >> rescale: one GEMM per batch, V is k-major.
+void einsum_bsht_btc_bshc(const int64_t *A, const int64_t *B, int64_t *C, int64_t rescale,
+                          int Bsz, int S, int H, int T, int Cdim)
+{
+    const char *name = "einsum_bsht_btc_bshc";
+    if (!zk::dims_ok(name, { Bsz, S, H, T, Cdim }, rescale)) return;
+    if ((long)Bsz * S * H * Cdim == 0) return;
+    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    zk::GemmDesc d;
+    d.A = A; d.lda = T; d.sA = (long)S * H * T;
+    d.B = B; d.b32 = 0; d.ldbn = 1; d.ldbk = Cdim; d.sB = (long)T * Cdim;
+    d.C = C; d.R = nullptr; d.ldc = Cdim; d.sC = (long)S * H * Cdim;
+    d.G = Bsz; d.M = S * H; d.N = Cdim; d.K = T;
+    d.shift = (int)rescale; d.init = rescale / 2; d.a_rs = 1; d.b_rs = 1;
+    zk::gemm_dispatch(name, d);
+}
+
+// out[b,s,h,d] = (sum_c A[b,s,h,c] * W[h,d,c]) >> rescale (no rounding term): one GEMM per head.
+void einsum_bshc_hdc_bshd(const int64_t *A, const int32_t *B, int64_t *C, int64_t rescale,
+                          int Bsz, int S, int H, int D, int Cdim)
+{
+    const char *name = "einsum_bshc_hdc_bshd";
+    if (!zk::dims_ok(name, { Bsz, S, H, D, Cdim }, rescale)) return;
+    if ((long)Bsz * S * H * D == 0) return;
+    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    zk::GemmDesc d;
+    d.A = A; d.lda = (long)H * Cdim; d.sA = Cdim;
+    d.B = B; d.b32 = 1; d.ldbn = Cdim; d.ldbk = 1; d.sB = (long)D * Cdim;
+    d.C = C; d.R = nullptr; d.ldc = (long)H * D; d.sC = D;
+    d.G = H; d.M = Bsz * S; d.N = D; d.K = Cdim;
+    d.shift = (int)rescale; d.init = 0; d.a_rs = 1; d.b_rs = 1;
+    zk::gemm_dispatch(name, d);
+}
+
+void zk_gemm_set_path(int path)
+{
+    if (path < 0 || path > 2) { zk::set_error(zk::kBadArgument, "zk_gemm_set_path: path %d outside [0,2]", path); return; }
+    zk::g_gemm_path = path;
+}
+
+int zk_gemm_get_path(void) { return zk::g_gemm_path; }
+
+void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b)
+{
+    if (path) *path = zk::g_last_path;
+    if (limbs_a) *limbs_a = zk::g_last_la;
+    if (limbs_b) *limbs_b = zk::g_last_lb;
+}
+
+}  // extern "C"

@@ -1,0 +1,217 @@
+// Fixed-point row softmax over the last dimension of [Bsz,S,H,T] int64 (Q19 truncating, Q21 rounding).
+//
+// Rows of up to 2048 elements are handled one row per wavefront: the row is read once with 16-byte loads
+// into registers, the maximum and the weight sum are 64-lane butterfly reductions, and the per-row divide
+// is a reciprocal multiply made exact by a remainder test.  HBM traffic is the algorithmic 16 bytes per
+// element (24 when the reference's write-back of the weights into the input is switched on).
+// Longer rows use one workgroup per row and three passes.
+//
+// Arithmetic follows inference/int64_gemm.cu:684-746 (Q19) and :605-659 (Q21).
+#include "common.h"
+#include "../../include/int64gemm.h"
+
+namespace zk {
+
+static bool g_softmax_clobber = false;
+
+struct __attribute__((aligned(16))) i64x2s { int64_t x, y; };
+
+template <int Q>
+__device__ __forceinline__ int64_t smx_weight(int64_t x, int64_t rmax, const int64_t *lut)
+{
+    if (Q == 19) {
+        uint64_t d = (uint64_t)rmax - (uint64_t)x;                 // >= 0 by construction
+        if (d > ((uint64_t)64 << 19)) return 0;
+        uint64_t y = (d * 756388ull) >> 19;                        // d <= 2^25: the product is below 2^45
+        uint64_t k = y >> 19;
+        uint64_t f = y & 0x7FFFF;
+        int64_t t = lut[f >> 11];
+        return k >= 64 ? 0 : (t >> (int)k);
+    } else {
+        int64_t d = (int64_t)((uint64_t)x - (uint64_t)rmax);       // <= 0 unless the subtraction wrapped
+        if (d < -((int64_t)64 << 21)) return 0;
+        int64_t y = (int64_t)((uint64_t)d * 3025551ull + (1ull << 20)) >> 21;
+        int64_t ny = (int64_t)(0 - (uint64_t)y);
+        int64_t k = ny >> 21;
+        int64_t f = ny & 0x1FFFFF;
+        int64_t t = lut[f >> 13];
+        if (k >= 64) return 0;
+        return k < 0 ? (t >> 63) : (t >> (int)k);
+    }
+}
+
+// Per-row divide.  fast: 2^12 <= s < 2^52 (true for every row whose maximum has weight LUT[0] = 2^Q).
+template <int Q>
+__device__ __forceinline__ int64_t smx_norm(int64_t w, int64_t s, double inv, bool fast)
+{
+    int64_t num = (int64_t)((uint64_t)w << Q);
+    if (Q == 21) num = (int64_t)((uint64_t)num + (uint64_t)(s / 2));
+    if (fast && w >= 0 && w < ((int64_t)1 << 30)) return (int64_t)udiv_by_inv((uint64_t)num, (uint64_t)s, inv);
+    return s ? tdiv64(num, s) : 0;
+}
+
+constexpr int kSmxThreads = 256;
+
+// One row per wavefront; EPL = elements per lane (even).  VEC: T is even and the pointers are 16-byte aligned.
+template <int Q, int EPL, bool VEC>
+__global__ __launch_bounds__(kSmxThreads) void softmax_wave_kernel(int64_t *__restrict__ R, int64_t *__restrict__ C,
+                                                                   const int64_t *__restrict__ lut_g, long rows, int T,
+                                                                   int clobber)
+{
+    __shared__ int64_t lut[256];
+    lut[threadIdx.x] = lut_g[threadIdx.x];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * (kSmxThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    int64_t *x = R + row * T;
+    int64_t *c = C + row * T;
+
+    int64_t v[EPL];
+    int64_t rmax = INT64_MIN;
+#pragma unroll
+    for (int j = 0; j < EPL / 2; j++) {
+        int idx = (j * 64 + lane) * 2;
+        if (VEC) {
+            if (idx < T) {
+                i64x2s p = *reinterpret_cast<const i64x2s *>(x + idx);
+                v[2 * j] = p.x;
+                v[2 * j + 1] = p.y;
+                rmax = p.x > rmax ? p.x : rmax;
+                rmax = p.y > rmax ? p.y : rmax;
+            }
+        } else {
+            if (idx < T) { v[2 * j] = x[idx]; rmax = v[2 * j] > rmax ? v[2 * j] : rmax; }
+            if (idx + 1 < T) { v[2 * j + 1] = x[idx + 1]; rmax = v[2 * j + 1] > rmax ? v[2 * j + 1] : rmax; }
+        }
+    }
+    rmax = wave_max_i64(rmax);
+
+    uint64_t sum = 0;
+#pragma unroll
+    for (int j = 0; j < EPL; j++) {
+        int idx = ((j >> 1) * 64 + lane) * 2 + (j & 1);
+        if (idx < T) {
+            v[j] = smx_weight<Q>(v[j], rmax, lut);
+            sum += (uint64_t)v[j];
+        }
+    }
+    const int64_t s = (int64_t)wave_sum_u64(sum);
+    const bool fast = s >= ((int64_t)1 << 12) && s < ((int64_t)1 << 52);
+    const double inv = fast ? 1.0 / (double)s : 0.0;
+
+#pragma unroll
+    for (int j = 0; j < EPL / 2; j++) {
+        int idx = (j * 64 + lane) * 2;
+        if (VEC) {
+            if (idx < T) {
+                i64x2s w, o;
+                w.x = v[2 * j];
+                w.y = v[2 * j + 1];
+                o.x = smx_norm<Q>(w.x, s, inv, fast);
+                o.y = smx_norm<Q>(w.y, s, inv, fast);
+                *reinterpret_cast<i64x2s *>(c + idx) = o;
+                if (clobber) *reinterpret_cast<i64x2s *>(x + idx) = w;
+            }
+        } else {
+            if (idx < T) {
+                c[idx] = smx_norm<Q>(v[2 * j], s, inv, fast);
+                if (clobber) x[idx] = v[2 * j];
+            }
+            if (idx + 1 < T) {
+                c[idx + 1] = smx_norm<Q>(v[2 * j + 1], s, inv, fast);
+                if (clobber) x[idx + 1] = v[2 * j + 1];
+            }
+        }
+    }
+}
+
+// One row per workgroup, any T: pass 1 maximum, pass 2 weights (staged in C) and their sum, pass 3 divide.
+// Each thread re-reads only what it wrote itself, so the staging needs no fence.
+template <int Q>
+__global__ __launch_bounds__(kSmxThreads) void softmax_block_kernel(int64_t *__restrict__ R, int64_t *__restrict__ C,
+                                                                    const int64_t *__restrict__ lut_g, int T, int clobber)
+{
+    __shared__ int64_t lut[256];
+    __shared__ int64_t red[kSmxThreads / 64];
+    lut[threadIdx.x] = lut_g[threadIdx.x];
+    const long row = blockIdx.x;
+    int64_t *x = R + row * T;
+    int64_t *c = C + row * T;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    int64_t rmax = INT64_MIN;
+    for (int i = threadIdx.x; i < T; i += kSmxThreads) { int64_t a = x[i]; rmax = a > rmax ? a : rmax; }
+    rmax = wave_max_i64(rmax);
+    if (lane == 0) red[wave] = rmax;
+    __syncthreads();
+    rmax = red[0];
+#pragma unroll
+    for (int w = 1; w < kSmxThreads / 64; w++) rmax = red[w] > rmax ? red[w] : rmax;
+    __syncthreads();
+
+    uint64_t sum = 0;
+    for (int i = threadIdx.x; i < T; i += kSmxThreads) {
+        int64_t w = smx_weight<Q>(x[i], rmax, lut);
+        c[i] = w;
+        if (clobber) x[i] = w;
+        sum += (uint64_t)w;
+    }
+    sum = wave_sum_u64(sum);
+    if (lane == 0) red[wave] = (int64_t)sum;
+    __syncthreads();
+    uint64_t tot = 0;
+#pragma unroll
+    for (int w = 0; w < kSmxThreads / 64; w++) tot += (uint64_t)red[w];
+    const int64_t s = (int64_t)tot;
+    const bool fast = s >= ((int64_t)1 << 12) && s < ((int64_t)1 << 52);
+    const double inv = fast ? 1.0 / (double)s : 0.0;
+    for (int i = threadIdx.x; i < T; i += kSmxThreads) c[i] = smx_norm<Q>(c[i], s, inv, fast);
+}
+
+template <int Q, int EPL>
+static void launch_wave(int64_t *R, int64_t *C, const int64_t *lut, long rows, int T, bool vec, int clobber)
+{
+    long blocks = (rows + (kSmxThreads / 64) - 1) / (kSmxThreads / 64);
+    if (vec)
+        softmax_wave_kernel<Q, EPL, true><<<dim3((unsigned)blocks), dim3(kSmxThreads), 0, 0>>>(R, C, lut, rows, T, clobber);
+    else
+        softmax_wave_kernel<Q, EPL, false><<<dim3((unsigned)blocks), dim3(kSmxThreads), 0, 0>>>(R, C, lut, rows, T, clobber);
+}
+
+template <int Q>
+static void launch_softmax(const char *name, int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int H, int T)
+{
+    if (Bsz < 0 || S < 0 || H < 0 || T < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
+    long rows = (long)Bsz * S * H;
+    if (rows == 0 || T == 0) return;
+    if (!R || !C || !lut) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    if (rows > 0x7FFFFFFFL) { set_error(kUnsupportedSize, "%s: more than 2^31-1 rows", name); return; }
+    int clobber = g_softmax_clobber ? 1 : 0;
+    bool vec = (T % 2 == 0) && ((((uintptr_t)R | (uintptr_t)C) & 15) == 0);
+    if (T <= 128) launch_wave<Q, 2>(R, C, lut, rows, T, vec, clobber);
+    else if (T <= 256) launch_wave<Q, 4>(R, C, lut, rows, T, vec, clobber);
+    else if (T <= 512) launch_wave<Q, 8>(R, C, lut, rows, T, vec, clobber);
+    else if (T <= 1024) launch_wave<Q, 16>(R, C, lut, rows, T, vec, clobber);
+    else if (T <= 2048) launch_wave<Q, 32>(R, C, lut, rows, T, vec, clobber);
+    else softmax_block_kernel<Q><<<dim3((unsigned)rows), dim3(kSmxThreads), 0, 0>>>(R, C, lut, T, clobber);
+    check_launch(name);
+}
+
+}  // namespace zk
+
+extern "C" {
+
+void softmax_q19(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int H, int T)
+{
+    zk::launch_softmax<19>("softmax_q19", R, C, lut, Bsz, S, H, T);
+}
+
+void softmax_q21(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int H, int T)
+{
+    zk::launch_softmax<21>("softmax_q21", R, C, lut, Bsz, S, H, T);
+}
+
+void zk_softmax_clobber_input(int on) { zk::g_softmax_clobber = on != 0; }
+
+}  // extern "C"

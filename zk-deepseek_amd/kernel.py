@@ -1,0 +1,297 @@
+"""Python operator API over libint64gemm.so for AMD MI355X.
+
+Same module name, function names, argument order and return values as the reference's
+inference/kernel.py:341-688, so `from kernel import ...` in the reference's model.py
+(inference/model.py:13-15) resolves against this file unchanged.  PyTorch is used only to
+allocate outputs and hand device pointers to the C ABI (include/int64gemm.h).
+
+Differences from the reference, all deliberate:
+  * the RMS statistic is computed on the device (one launch) instead of one `.item()` sync per
+    element (inference/kernel.py:477-494, 539-542);
+  * every call checks the library's error channel and raises RuntimeError instead of returning
+    uninitialised tensors;
+  * `act_quant`, `weight_dequant`, `fp8_gemm` (Triton fp8 leftovers that no int64 layer reaches) are
+    importable names that raise NotImplementedError.
+There is no CPU fallback: if the shared object is missing, importing this module raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _find_library():
+    # the reference loads "./libint64gemm.so" relative to the working directory (inference/kernel.py:206)
+    for cand in (os.path.join(os.getcwd(), "libint64gemm.so"), os.path.join(_HERE, "libint64gemm.so")):
+        if os.path.exists(cand):
+            return cand
+    raise ImportError(
+        "libint64gemm.so not found in the working directory or next to kernel.py; "
+        "build it with `python zk-deepseek_amd/build.py` (hipcc, gfx950). There is no CPU fallback.")
+
+
+LIB_PATH = _find_library()
+lib = ctypes.CDLL(LIB_PATH)
+
+_vp, _ll, _ci = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
+
+lib.int64_64_bmm_broadcast_launcher.argtypes = [_vp, _vp, _vp, _vp, _ll, _ll, _ll, _ci, _ci, _ci, _ci]
+lib.int64_32_bmm_broadcast_launcher.argtypes = [_vp, _vp, _vp, _vp, _ll, _ll, _ll, _ci, _ci, _ci, _ci]
+lib.complex_int64_mul.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _ci]
+lib.rms_norm_32.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci]
+lib.rms_norm_64.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci]
+for _n in ("einsum_bshd_hdc_bshc", "einsum_bshc_btc_bsht", "einsum_bsht_btc_bshc", "einsum_bshc_hdc_bshd"):
+    getattr(lib, _n).argtypes = [_vp, _vp, _vp, _ll, _ci, _ci, _ci, _ci, _ci]
+lib.softmax_q21.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _ci]
+lib.softmax_q19.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _ci]
+for _n in ("softmax_init_q21", "softmax_init_q19", "silu_init_q25", "silu_init_q23"):
+    getattr(lib, _n).argtypes = [_vp]
+for _n in ("silu_q25", "sigmoid_q25", "silu_q23", "sigmoid_q23"):
+    getattr(lib, _n).argtypes = [_vp, _vp, _vp, _ci, _ci, _ci]
+for _n in ("bf16_to_int32_2d", "float32_to_int64_2d"):
+    getattr(lib, _n).argtypes = [_vp, _vp, _ci, _ci, _ci]
+lib.wkv_b_bf16_to_int32.argtypes = [_vp, _vp, _ci, _ci]
+# additions without a reference counterpart
+lib.rms_stat_int64.argtypes = [_vp, _vp, _ci, _ci, _ll, _ll]
+lib.rms_norm_fused_32.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
+lib.rms_norm_fused_64.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
+lib.zk_last_error.restype = _ci
+lib.zk_last_error_string.restype = ctypes.c_char_p
+lib.zk_softmax_clobber_input.argtypes = [_ci]
+lib.zk_gemm_set_path.argtypes = [_ci]
+lib.zk_gemm_get_path.restype = _ci
+lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
+lib.zk_timer_stop_ms.restype = ctypes.c_float
+
+
+def _check(what):
+    code = lib.zk_last_error()
+    if code != 0:
+        msg = lib.zk_last_error_string().decode()
+        lib.zk_clear_error()
+        raise RuntimeError("%s failed (code %d): %s" % (what, code, msg))
+
+
+def gemm_last_plan():
+    """(path, limbs_a, limbs_b) of the last GEMM-shaped call: path 1 = VALU, 2 = i8 MFMA."""
+    p, a, b = _ci(), _ci(), _ci()
+    lib.zk_gemm_last_plan(ctypes.byref(p), ctypes.byref(a), ctypes.byref(b))
+    return p.value, a.value, b.value
+
+
+def act_quant(*args, **kwargs):
+    raise NotImplementedError("act_quant belongs to the fp8 path, which the int64 model never reaches")
+
+
+def weight_dequant(*args, **kwargs):
+    raise NotImplementedError("weight_dequant belongs to the offline fp8 checkpoint converter")
+
+
+def fp8_gemm(*args, **kwargs):
+    raise NotImplementedError("fp8_gemm belongs to the fp8 path, which the int64 model never reaches")
+
+
+def int64_bmm_broadcast(A: torch.Tensor, B: torch.Tensor, a_rescale, b_rescale, c_rescale):
+    """(B, M, K) x (N, K) -> quotient C and remainder R, both (B, M, N) int64."""
+    assert A.dtype == torch.int64
+    assert A.is_cuda and B.is_cuda
+    Bdim, M, K = A.shape
+    N, K2 = B.shape
+    assert K2 == K
+
+    C = torch.empty((Bdim, M, N), dtype=torch.int64, device=A.device)
+    R = torch.empty((Bdim, M, N), dtype=torch.int64, device=A.device)
+
+    if B.dtype == torch.int64:
+        lib.int64_64_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), R.data_ptr(),
+                                            a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
+    elif B.dtype == torch.int32:
+        lib.int64_32_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), R.data_ptr(),
+                                            a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
+    else:
+        raise TypeError(f"Unsupported B type: {B.dtype}")
+    _check("int64_bmm_broadcast")
+    return (C, R)
+
+
+def complex_int64_mul_broadcast(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """Complex multiply in Q42; A [batch, seq, heads, headDim, 2], B [1, seq, 1, headDim, 2]."""
+    assert A.dtype == torch.int64 and B.dtype == torch.int64
+    assert A.is_cuda and B.is_cuda
+    batch, seqLen, head, headDim = A.shape[0], A.shape[1], A.shape[2], A.shape[3]
+    C = torch.empty(A.shape, dtype=torch.int64, device=A.device)
+    lib.complex_int64_mul(A.data_ptr(), B.data_ptr(), C.data_ptr(), batch, seqLen, head, headDim)
+    _check("complex_int64_mul_broadcast")
+    return C
+
+
+def einsum_bshd_hdc_bshc(A: torch.Tensor, B: torch.Tensor, rescale) -> torch.Tensor:
+    assert A.shape[2] == B.shape[0] and A.shape[3] == B.shape[1]
+    assert A.is_cuda and B.is_cuda
+    assert A.dtype == torch.int64 and B.dtype == torch.int32
+    Batch, S, H, D = A.shape
+    Cp = B.shape[2]
+    C = torch.empty([Batch, S, H, Cp], dtype=torch.int64, device=A.device)
+    lib.einsum_bshd_hdc_bshc(A.data_ptr(), B.data_ptr(), C.data_ptr(), rescale, Batch, S, H, D, Cp)
+    _check("einsum_bshd_hdc_bshc")
+    return C
+
+
+def einsum_bshc_btc_bsht(A: torch.Tensor, B: torch.Tensor, rescale) -> torch.Tensor:
+    Bsz, S, H, Cdim = A.shape
+    T = B.shape[1]
+    assert Bsz == B.shape[0] and Cdim == B.shape[2]
+    assert A.is_cuda and B.is_cuda
+    assert A.dtype == torch.int64 and B.dtype == torch.int64
+    C = torch.empty([Bsz, S, H, T], dtype=torch.int64, device=A.device)
+    lib.einsum_bshc_btc_bsht(A.data_ptr(), B.data_ptr(), C.data_ptr(), rescale, Bsz, S, H, T, Cdim)
+    _check("einsum_bshc_btc_bsht")
+    return C
+
+
+def einsum_bsht_btc_bshc(A: torch.Tensor, B: torch.Tensor, rescale) -> torch.Tensor:
+    Bsz, S, H, T = A.shape
+    Cdim = B.shape[2]
+    assert Bsz == B.shape[0] and T == B.shape[1]
+    assert A.is_cuda and B.is_cuda
+    assert A.dtype == torch.int64 and B.dtype == torch.int64
+    C = torch.empty([Bsz, S, H, Cdim], dtype=torch.int64, device=A.device)
+    lib.einsum_bsht_btc_bshc(A.data_ptr(), B.data_ptr(), C.data_ptr(), rescale, Bsz, S, H, T, Cdim)
+    _check("einsum_bsht_btc_bshc")
+    return C
+
+
+def einsum_bshc_hdc_bshd(A: torch.Tensor, B: torch.Tensor, rescale) -> torch.Tensor:
+    Bsz, S, H, Cdim = A.shape
+    D = B.shape[1]
+    assert H == B.shape[0] and Cdim == B.shape[2]
+    assert A.is_cuda and B.is_cuda
+    assert A.dtype == torch.int64 and B.dtype == torch.int32
+    C = torch.empty([Bsz, S, H, D], dtype=torch.int64, device=A.device)
+    lib.einsum_bshc_hdc_bshd(A.data_ptr(), B.data_ptr(), C.data_ptr(), rescale, Bsz, S, H, D, Cdim)
+    _check("einsum_bshc_hdc_bshd")
+    return C
+
+
+def int64_RMS0(A: torch.Tensor, eps: int, dim: int) -> int:
+    """isqrt((eps + sum a^2) // dim) of a 1-D int64 tensor, as a Python int."""
+    assert A.dtype == torch.int64
+    assert A.ndim == 1
+    assert A.is_cuda
+    out = torch.empty((1,), dtype=torch.int64, device=A.device)
+    A = A.contiguous()
+    lib.rms_stat_int64(A.data_ptr(), out.data_ptr(), 1, A.shape[0], eps, dim)
+    _check("int64_RMS0")
+    return int(out.item())
+
+
+# The reference keeps one 500-row host buffer and returns it whole (rows >= M keep older values);
+# callers slice it (inference/kernel.py:525-526, 550).  The device twin is allocated on first use.
+rms = torch.zeros((500,), dtype=torch.int64, device="cpu")
+rms_gpu = None
+
+
+def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim):
+    """C = floor(A * W / rms) per row, rms = isqrt((eps + sum a^2) // dim).  Returns (C, rms buffer)."""
+    global rms, rms_gpu
+    assert A.dtype == torch.int64
+    assert A.is_cuda and W.is_cuda
+    assert A.ndim == 2
+    M, N = A.shape
+    assert M <= rms.shape[0], "the rms buffer holds 500 rows, as in the reference"
+    if rms_gpu is None or rms_gpu.device != A.device:
+        rms_gpu = torch.zeros((500,), dtype=torch.int64, device=A.device)
+    C = torch.empty((M, N), dtype=torch.int64, device=A.device)
+    if W.dtype == torch.int32:
+        lib.rms_norm_fused_32(A.data_ptr(), W.data_ptr(), rms_gpu.data_ptr(), C.data_ptr(), M, N, eps, dim)
+    else:
+        assert W.dtype == torch.int64
+        lib.rms_norm_fused_64(A.data_ptr(), W.data_ptr(), rms_gpu.data_ptr(), C.data_ptr(), M, N, eps, dim)
+    _check("RMS_Norm_int64")
+    rms[:M] = rms_gpu[:M].cpu()
+    return (C, rms)
+
+
+def saveTensor(fileName, t):
+    """Raw C-order little-endian bytes, the witness format the proving side reads back."""
+    t = t.detach()
+    if t.device.type != "cpu":
+        t = t.cpu()
+    t = t.contiguous()
+    with open(fileName, "wb") as f:
+        f.write(t.numpy().tobytes(order="C"))
+
+
+LOG_TABLE_SIZE = 8
+EXP2_FRAC_LUT_Q21 = None
+EXP2_FRAC_LUT_Q19 = None
+EXP2_FRAC_LUT_Q25 = None
+EXP2_FRAC_LUT_Q23 = None
+
+
+def _host_table(init_fn):
+    table = torch.zeros((2 ** LOG_TABLE_SIZE,), dtype=torch.int64, device="cpu")
+    init_fn(table.data_ptr())
+    return table
+
+
+def softmax_init_q21():
+    global EXP2_FRAC_LUT_Q21
+    EXP2_FRAC_LUT_Q21 = _host_table(lib.softmax_init_q21).cuda()
+
+
+def softmax_init_q19():
+    global EXP2_FRAC_LUT_Q19
+    EXP2_FRAC_LUT_Q19 = _host_table(lib.softmax_init_q19).cuda()
+
+
+def silu_init_q25():
+    global EXP2_FRAC_LUT_Q25
+    EXP2_FRAC_LUT_Q25 = _host_table(lib.silu_init_q25).cuda()
+
+
+def silu_init_q23():
+    global EXP2_FRAC_LUT_Q23
+    EXP2_FRAC_LUT_Q23 = _host_table(lib.silu_init_q23).cuda()
+
+
+def _softmax(fn, name, R, C, lut):
+    assert R.is_cuda and C.is_cuda
+    assert lut is not None, "call the matching *_init_* first"
+    Bsz, S, H, T = R.shape
+    fn(R.data_ptr(), C.data_ptr(), lut.data_ptr(), Bsz, S, H, T)
+    _check(name)
+
+
+def softmax_q21(R: torch.Tensor, C: torch.Tensor):
+    _softmax(lib.softmax_q21, "softmax_q21", R, C, EXP2_FRAC_LUT_Q21)
+
+
+def softmax_q19(R: torch.Tensor, C: torch.Tensor):
+    _softmax(lib.softmax_q19, "softmax_q19", R, C, EXP2_FRAC_LUT_Q19)
+
+
+def _act(fn, name, R, C, lut):
+    assert R.is_cuda and C.is_cuda
+    assert lut is not None, "call the matching *_init_* first"
+    Bsz, S, Dim = R.shape
+    fn(R.data_ptr(), C.data_ptr(), lut.data_ptr(), Bsz, S, Dim)
+    _check(name)
+
+
+def silu_q25(R: torch.Tensor, C: torch.Tensor):
+    _act(lib.silu_q25, "silu_q25", R, C, EXP2_FRAC_LUT_Q25)
+
+
+def sigmoid_q25(R: torch.Tensor, C: torch.Tensor):
+    _act(lib.sigmoid_q25, "sigmoid_q25", R, C, EXP2_FRAC_LUT_Q25)
+
+
+def silu_q23(R: torch.Tensor, C: torch.Tensor):
+    _act(lib.silu_q23, "silu_q23", R, C, EXP2_FRAC_LUT_Q23)
+
+
+def sigmoid_q23(R: torch.Tensor, C: torch.Tensor):
+    _act(lib.sigmoid_q23, "sigmoid_q23", R, C, EXP2_FRAC_LUT_Q23)
