@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the witness-generation hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+Prints ONE JSON line.  `value` is the int64 GEMM throughput (Gmac/s) of BASELINE config 4
+(512 x 7168 against W[18432,7168], config-1 operand ranges, shift 29) through the C ABI with operands
+resident in HBM; one step = one call of int64_64_bmm_broadcast_launcher.  The same line carries the
+other shapes the metric names (config-1 GEMM, full-range config 4, softmax / SiLU / sigmoid / RMSNorm
+HBM GB/s) under "extra", the roofline of the dominant kernel, and a CPU baseline timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (os.path.join(ROOT, "zk-deepseek_amd"),):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+I8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,cpu (default all)")
+    return ap.parse_args()
+
+
+def randint(gen, lo, hi, shape, dtype=None):
+    import torch
+    return torch.randint(lo, hi, shape, generator=gen, dtype=dtype or torch.int64)
+
+
+def full_range(gen, shape):
+    import torch
+    hi = torch.randint(-(1 << 31), 1 << 31, shape, generator=gen, dtype=torch.int64)
+    lo = torch.randint(0, 1 << 32, shape, generator=gen, dtype=torch.int64)
+    return (hi << 32) | lo
+
+
+def timed(K, fn, steps, warmup):
+    """average milliseconds per call, measured with HIP events on the null stream (where the library launches)"""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    K.lib.zk_timer_start()
+    for _ in range(steps):
+        fn()
+    ms = K.lib.zk_timer_stop_ms()
+    torch.cuda.synchronize()
+    return ms / steps
+
+
+def gemm_leg(K, A, W, c, steps, warmup):
+    import torch
+    Bd, M, Kd = A.shape
+    N = W.shape[0]
+    C = torch.empty((Bd, M, N), dtype=torch.int64, device="cuda")
+    R = torch.empty((Bd, M, N), dtype=torch.int64, device="cuda")
+    fn = K.lib.int64_64_bmm_broadcast_launcher if W.dtype == torch.int64 else K.lib.int64_32_bmm_broadcast_launcher
+
+    def call():
+        fn(A.data_ptr(), W.data_ptr(), C.data_ptr(), R.data_ptr(), 1, 1, c, Bd, M, Kd, N)
+
+    ms = timed(K, call, steps, warmup)
+    K._check("gemm bench")
+    path, la, lb = K.gemm_last_plan()
+    macs = Bd * M * N * Kd
+    return {"ms": ms, "gmacs": macs / ms / 1e6, "macs": macs, "path": {1: "valu", 2: "mfma_i8"}.get(path, "?"),
+            "limbs_a": la, "limbs_b": lb}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); --gpus must be 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import kernel as K
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    legs = set(args.only.split(",")) if args.only else {"gemm", "extra", "cpu"}
+    if args.no_cpu:
+        legs.discard("cpu")
+    gen = torch.Generator(device="cpu").manual_seed(4000)
+    extra = {}
+
+    # ---------------- headline: config 4 GEMM ----------------------------------------------
+    M, Kd, N, c = 512, 7168, 18432, 29
+    A_h = randint(gen, -(1 << 20), 1 << 20, (1, M, Kd))
+    W_h = randint(gen, -(1 << 16), 1 << 16, (N, Kd))
+    A, W = A_h.cuda(), W_h.cuda()
+    # the timed region proper: W warmup calls, then exactly K steps between synchronisations
+    Cb = torch.empty((1, M, N), dtype=torch.int64, device="cuda")
+    Rb = torch.empty((1, M, N), dtype=torch.int64, device="cuda")
+
+    def step():
+        K.lib.int64_64_bmm_broadcast_launcher(A.data_ptr(), W.data_ptr(), Cb.data_ptr(), Rb.data_ptr(),
+                                              1, 1, c, 1, M, Kd, N)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    K.lib.zk_timer_start()
+    for _ in range(args.steps):
+        step()
+    ev_ms = K.lib.zk_timer_stop_ms()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    K._check("config-4 GEMM")
+    path, la, lb = K.gemm_last_plan()
+    macs = M * N * Kd
+    ms_per_step = wall_ms / args.steps
+    kern_ms = ev_ms / args.steps
+    value = macs / ms_per_step / 1e6                     # Gmac/s
+
+    if path == 2:
+        pairs = la * lb
+        ops = 2.0 * pairs * macs                         # i8 multiply-adds issued as MFMA, counted as 2 ops
+        achieved = ops / (kern_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": I8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": achieved / I8_MFMA_PEAK_TOPS, "traffic": None,
+                    "note": "i8 MFMA ops = 2 * limbs_a * limbs_b * M*N*K (%dx%d limb pairs per int64 MAC); "
+                            "duration = HIP events over the whole launcher" % (la, lb)}
+    else:
+        achieved = macs / (kern_ms * 1e-3) / 1e12
+        roofline = {"bound": "valu", "achieved": achieved, "peak": None, "unit": "Tmac/s", "frac": None,
+                    "traffic": None, "note": "VALU 64-bit multiply-add path; no published peak"}
+
+    if "extra" in legs:
+        # config 1 (M=16): weight-bandwidth bound
+        g1 = torch.Generator(device="cpu").manual_seed(1000)
+        A1 = randint(g1, -(1 << 20), 1 << 20, (1, 16, 7168)).cuda()
+        W1 = randint(g1, -(1 << 16), 1 << 16, (576, 7168)).cuda()
+        extra["gemm_config1_16x7168x576"] = gemm_leg(K, A1, W1, 29, 50, 5)
+        # config 4, full-range operands (two's-complement wraparound)
+        g4 = torch.Generator(device="cpu").manual_seed(4001)
+        Af = full_range(g4, (1, M, Kd)).cuda()
+        Wf = full_range(g4, (N, Kd)).cuda()
+        extra["gemm_config4_full_range"] = gemm_leg(K, Af, Wf, 29, max(3, args.steps // 4), 1)
+        del Af, Wf
+        # real-model operand widths: Q31 activations (|x| < 2^37), int32 weights
+        Am = randint(g4, -(1 << 37), 1 << 37, (1, M, Kd)).cuda()
+        Wm = randint(g4, -(1 << 31), 1 << 31, (N, Kd)).to(torch.int32).cuda()
+        extra["gemm_config4_q31_x_int32"] = gemm_leg(K, Am, Wm, 30, max(3, args.steps // 2), 1)
+        del Am, Wm
+        # other instruction path on the headline shape, for the comparison
+        K.lib.zk_gemm_set_path(1 if path == 2 else 2)
+        extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1)
+        K.lib.zk_gemm_set_path(0)
+
+        # memory-bound kernels, 16 algorithmic bytes per element
+        K.softmax_init_q19()
+        K.silu_init_q23()
+
+        def hbm(name, fn, nelem, bytes_per_elem=16.0, extra_bytes=0.0, steps=30):
+            ms = timed(K, fn, steps, 3)
+            K._check(name)
+            gbs = (nelem * bytes_per_elem + extra_bytes) / (ms * 1e-3) / 1e9
+            extra[name] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS, "elements": nelem}
+
+        for S in (1024, 4096):
+            g3 = torch.Generator(device="cpu").manual_seed(3000 + S)
+            x = randint(g3, -(6 << 19), 6 << 19, (1, S, 128, 1024))
+            if S == 1024:
+                x += torch.full((S, 1024), -(64 << 36), dtype=torch.int64).triu_(1).unsqueeze(1)
+            R = x.cuda()
+            del x
+            Cs = torch.empty_like(R)
+            hbm("softmax_q19_1x%dx128x1024" % S,
+                lambda: K.lib.softmax_q19(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q19.data_ptr(), 1, S, 128, 1024),
+                R.numel(), steps=10)
+            del R, Cs
+        for S in (512, 8192):
+            g2 = torch.Generator(device="cpu").manual_seed(2300 + S)
+            R = randint(g2, -(16 << 23), 16 << 23, (1, S, 18432)).cuda()
+            Cs = torch.empty_like(R)
+            for nm, fn in (("silu_q23", K.lib.silu_q23), ("sigmoid_q23", K.lib.sigmoid_q23)):
+                hbm("%s_1x%dx18432" % (nm, S),
+                    lambda fn=fn: fn(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q23.data_ptr(), 1, S, 18432),
+                    R.numel(), steps=20)
+            del R, Cs
+        g6 = torch.Generator(device="cpu").manual_seed(600)
+        for Mr in (500, 16384):
+            Ar = randint(g6, -(1 << 37), 1 << 37, (Mr, 7168)).cuda()
+            Wr = randint(g6, 1 << 18, 1 << 20, (7168,)).to(torch.int32).cuda()
+            rr = torch.empty((Mr,), dtype=torch.int64, device="cuda")
+            Cr = torch.empty_like(Ar)
+            hbm("rmsnorm_fused_%dx7168" % Mr,
+                lambda: K.lib.rms_norm_fused_32(Ar.data_ptr(), Wr.data_ptr(), rr.data_ptr(), Cr.data_ptr(), Mr, 7168, 1, 7168),
+                Ar.numel(), extra_bytes=4.0 * 7168 + 8.0 * Mr, steps=20)
+            del Ar, Cr
+
+    cpu_baseline = None
+    if "cpu" in legs:
+        cpu_baseline = cpu_leg(A_h, W_h, c)
+
+    out = {
+        "metric": "int64 GEMM Gmac/s @7168x576 & 18432x7168 + softmax/SiLU HBM GB/s, 1 MI355X",
+        "value": value, "unit": "Gmac/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "config4: int64 GEMM Y[512,18432] = X[512,7168] @ W[18432,7168]^T, int64 W, "
+                               "X in [-2^20,2^20), W in [-2^16,2^16), c_rescale=29, C and R written",
+                   "path": {1: "valu", 2: "mfma_i8"}.get(path, "?"), "limbs_a": la, "limbs_b": lb,
+                   "kernel_ms_hip_events": kern_ms},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+
+
+def cpu_leg(A_h, W_h, c):
+    """The reference's CPU path for a Linear layer is torch's int64 matmul on CPU tensors followed by the shift
+    (the generic branch of `linear`, inference/model.py:179-181).  Timed on a column block of config 4 sized to
+    take roughly 10-30 s, with all host cores and with the reference's own 8 threads."""
+    import torch
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    omp = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    if omp > 0:
+        cores = min(cores, omp)
+    A2 = A_h[0]
+
+    def run(ncols, threads):
+        torch.set_num_threads(threads)
+        Wt = W_h[:ncols].T.contiguous()
+        t0 = time.perf_counter()
+        y = torch.matmul(A2, Wt) >> c
+        dt = time.perf_counter() - t0
+        return dt, y
+
+    dt, _ = run(16, cores)                                  # calibrate
+    rate = 512 * 7168 * 16 / dt
+    ncols = int(min(W_h.shape[0], max(64, (rate * 15.0) // (512 * 7168))))
+    dt, y = run(ncols, cores)
+    macs = 512 * 7168 * ncols
+    res = {"value": macs / dt / 1e9, "unit": "Gmac/s", "cores": cores, "kind": "reference",
+           "sample": "torch.matmul int64 on CPU then >> %d (the reference's F.linear CPU branch, model.py:179-181) on "
+                     "X[512,7168] x W[:%d,7168]^T of config 4, %.1f s" % (c, ncols, dt)}
+    if cores > 8:
+        dt8, _ = run(max(64, ncols // 2), 8)
+        res["value_8_threads"] = 512 * 7168 * max(64, ncols // 2) / dt8 / 1e9
+    return res
+
+
+if __name__ == "__main__":
+    main()

@@ -389,3 +389,23 @@ def test_rope(K, oracle, bits):
     Bt = rand_i64(rng, (1, 7, 1, 32, 2), 43)
     out = K.complex_int64_mul_broadcast(dev(A), dev(Bt))
     assert np.array_equal(host(out), oracle.complex_int64_mul_broadcast(A, Bt))
+
+
+def test_gemm_mfma_path_is_taken(K, oracle):
+    """the i8 MFMA path must really run (and report its digit counts) on the shapes it is meant for"""
+    rng = np.random.default_rng(42)
+    A = rand_i64(rng, (1, 64, 256), 20)
+    W = rand_i64(rng, (128, 256), 16)
+    K.lib.zk_gemm_set_path(2)
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    assert K.gemm_last_plan() == (2, 3, 3)
+    Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 29)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    A = rand_i64(rng, (1, 64, 256), 63)
+    W = rand_i64(rng, (128, 256), 63)
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    assert K.gemm_last_plan() == (2, 9, 9)
+    K.lib.zk_gemm_set_path(1)
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    assert K.gemm_last_plan() == (1, 0, 0)
+    K.lib.zk_gemm_set_path(0)

@@ -54,7 +54,7 @@ def build(force=False, verbose=True):
         for out in ex.map(_run, jobs):
             if verbose and out.strip():
                 print(out)
-    if jobs or not os.path.exists(LIB):
+    if jobs or not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(o) for o in objs):
         out = _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs)
         if verbose and out.strip():
             print(out)
