@@ -9,9 +9,13 @@
 // all pairs with the same i+j share one int32 accumulator tile, and the epilogue recombines the
 // NA+NB-1 diagonals with carries into the 128-bit sum before the shift.  Nothing is approximated.
 //
-// Operand tiles are converted on the fly: a thread loads 8 consecutive k of one row (64 bytes), splits them
-// into digits with v_perm_b32 byte transposes and stores each digit plane to LDS already in MFMA fragment
-// order (lane l of a fragment = row l%32, k-half l/32, 16 bytes), so the inner loop is ds_read_b128 + MFMA.
+// Operand tiles are converted on the fly: a thread gathers 8 elements of one row, splits them into digits with
+// v_perm_b32 byte transposes and stores each digit plane to LDS already in MFMA fragment order (lane l of a
+// fragment = row l%32, k-half l/32, 16 bytes), so the inner loop is ds_read_b128 + MFMA.
+// A dot product does not care about the order of k as long as both operands use the same one, so the 8
+// elements a thread owns are NOT consecutive: thread j of a row owns runs of RUN consecutive k spaced
+// RUN*OCTS apart.  Adjacent lanes then read adjacent 16-byte pieces and every 64-byte line of the tile is
+// fetched by exactly one load instruction.
 //
 // The digit counts are speculated from a cached or sampled range; the workgroups of the first tile row /
 // column track the exact min and max of everything they load, the launcher reads them back and reruns with
@@ -22,6 +26,19 @@
 #include <mutex>
 #include <set>
 #include <tuple>
+#include <type_traits>
+
+// Tuning knobs: MFMA depths (32 k each) per pipeline step by diagonal count, and how many vector-ALU
+// instructions of the digit split are scheduled behind each MFMA of a step's last depth.
+#ifndef ZK_VALU_PER_MFMA
+#define ZK_VALU_PER_MFMA 8
+#endif
+#ifndef ZK_PREFETCH
+#define ZK_PREFETCH 0
+#endif
+#ifndef ZK_KK
+#define ZK_KK(DD) 1
+#endif
 
 namespace zk {
 
@@ -38,6 +55,9 @@ struct MfmaParams {
     int tiles_m, tiles_n;
     unsigned long long *range;      // [minA, maxA, minB, maxB], order-preserving unsigned images of int64
     int verify_b_all_batches;       // B differs per batch: every batch's first tile row tracks its range
+    const unsigned char *a_planes;  // pre-split digits of A (planes variants only)
+    int a_msub, a_ksteps;           // 32-row groups and 32-k steps the planes were written for
+    int dbg;
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -114,7 +134,7 @@ __device__ __forceinline__ void mm_update(MinMax &r, int64_t v)
     r.hi = v > r.hi ? v : r.hi;
 }
 
-__device__ __forceinline__ void mm_publish(MinMax r, unsigned long long *slot)
+__device__ __forceinline__ MinMax mm_wave(MinMax r)
 {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -122,9 +142,18 @@ __device__ __forceinline__ void mm_publish(MinMax r, unsigned long long *slot)
         r.lo = ol < r.lo ? ol : r.lo;
         r.hi = oh > r.hi ? oh : r.hi;
     }
+    return r;
+}
+
+__device__ __forceinline__ void mm_publish(MinMax r, unsigned long long *slot)
+{
+    r = mm_wave(r);
+    // The slots only ever move one way, so a plain (possibly stale) read is enough to skip the atomic when this
+    // wave cannot improve them; that keeps thousands of waves from serialising on two addresses.
     if ((threadIdx.x & 63) == 0) {
-        atomicMin(slot, (unsigned long long)r.lo ^ kSignFlip);
-        atomicMax(slot + 1, (unsigned long long)r.hi ^ kSignFlip);
+        const unsigned long long lo = (unsigned long long)r.lo ^ kSignFlip, hi = (unsigned long long)r.hi ^ kSignFlip;
+        if (lo < __atomic_load_n(slot, __ATOMIC_RELAXED)) atomicMin(slot, lo);
+        if (hi > __atomic_load_n(slot + 1, __ATOMIC_RELAXED)) atomicMax(slot + 1, hi);
     }
 }
 
@@ -159,36 +188,158 @@ __global__ __launch_bounds__(256) void range_sample_kernel(MfmaParams p, int b32
     mm_publish(r, p.range + 2 * which);
 }
 
-// ---- the GEMM kernel -------------------------------------------------------------------------------
-// WM x WN 32x32 MFMA tiles per wave, 2x2 waves per workgroup: workgroup tile (64*WM) x (64*WN), k-step 32.
-template <int NA, int NB, int WM, int WN, bool B32, bool BKM>
-__global__ __launch_bounds__(256, 1) void gemm_mfma_kernel(MfmaParams p)
+// ---- element ownership ---------------------------------------------------------------------------
+// Within a pipeline step of BK = 8*OCTS k-values, thread j (0 <= j < OCTS) of a row owns elements
+//     k(e) = RUN*OCTS*(e / RUN) + RUN*j + e % RUN,   e = 0..7,
+// i.e. 8/RUN runs of RUN consecutive k.  RUN = 2 for int64 B (a run is one 16-byte load), 4 for int32 B.
+template <int RUN, int OCTS>
+__device__ __forceinline__ int owned_k(int j, int e) { return RUN * OCTS * (e / RUN) + RUN * j + e % RUN; }
+
+// Loads the 8 owned int64 elements of one row; `src` points at the row's first k of this step.
+template <int RUN, int OCTS>
+__device__ __forceinline__ void load_owned_i64(const int64_t *src, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
 {
-    constexpr int BM = 64 * WM, BN = 64 * WN;
+    if (row_ok && owned_k<RUN, OCTS>(j, 7) < k_left && vec) {
+#pragma unroll
+        for (int q = 0; q < 8 / RUN; q++) {
+#pragma unroll
+            for (int h = 0; h < RUN / 2; h++) {
+                const v4i t = *reinterpret_cast<const v4i *>(src + owned_k<RUN, OCTS>(j, q * RUN + 2 * h));
+                x[q * RUN + 2 * h] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
+                x[q * RUN + 2 * h + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int k = owned_k<RUN, OCTS>(j, e);
+            x[e] = (row_ok && k < k_left) ? src[k] : 0;
+        }
+    }
+}
+
+template <int RUN, int OCTS>
+__device__ __forceinline__ void load_owned_i32(const int32_t *src, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
+{
+    if (RUN == 4 && row_ok && owned_k<RUN, OCTS>(j, 7) < k_left && vec) {
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const v4i t = *reinterpret_cast<const v4i *>(src + owned_k<RUN, OCTS>(j, q * 4));
+#pragma unroll
+            for (int z = 0; z < 4; z++) x[q * 4 + z] = (int64_t)t[z];
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int k = owned_k<RUN, OCTS>(j, e);
+            x[e] = (row_ok && k < k_left) ? (int64_t)src[k] : 0;
+        }
+    }
+}
+
+// Byte offset, inside one operand region of an LDS stage (or of a plane step), of the 8 digit bytes that
+// thread j of `row` produces: 1 KB fragment blocks, lane slot = row%32 + 32*(k-half), 16 bytes per slot.
+__device__ __forceinline__ int frag_offset(int row, int j, int n_limbs, int substage_bytes)
+{
+    const int o4 = j & 3;
+    return (j >> 2) * substage_bytes + ((row >> 5) * n_limbs) * 1024 + ((row & 31) + 32 * (o4 >> 1)) * 16 + (o4 & 1) * 8;
+}
+
+// ---- A digit planes (pre-pass) ------------------------------------------------------------------
+// When A is reused by many column tiles it is split once, into digit planes stored in MFMA fragment order:
+// block (g, sub, ks32, i) of 1 KB holds digit i of rows [32*sub, 32*sub+32) for the 32 owned-k slots of MFMA
+// depth ks32, lane-major.  Rows >= M and k >= K are written as zero digits.  Each workgroup also leaves the
+// min and max of what it read in mm[2*block .. 2*block+1].
+template <int NA, int RUN, int KK>
+__global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned char *planes, int msub, int ksteps32,
+                                                       unsigned long long *mm)
+{
+    constexpr int OCTS = 4 * KK, ROWS = 256 / OCTS;
+    __shared__ MinMax red[4];
+    const int tid = threadIdx.x;
+    const int g = blockIdx.z, ks = blockIdx.x;
+    const int row = blockIdx.y * ROWS + tid / OCTS, j = tid % OCTS;
+    const int k0 = ks * (8 * OCTS);
+    const bool vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
+    int64_t x[8];
+    load_owned_i64<RUN, OCTS>(p.A + (long)g * p.sA + (long)row * p.lda + k0, j, row < p.M, p.K - k0, vec, x);
+    MinMax r = { INT64_MAX, INT64_MIN };
+#pragma unroll
+    for (int q = 0; q < 8; q++) mm_update(r, x[q]);
+    uint2 dg[NA];
+    limb_split8<NA>(x, dg);
+    // plane step layout: [g][sub][ks32][digit][1 KB]; a step of KK depths is contiguous per sub
+    unsigned char *dst = planes + (((long)g * msub + (row >> 5)) * ksteps32 + ks * KK + (j >> 2)) * (NA * 1024) +
+                         ((row & 31) + 32 * ((j & 3) >> 1)) * 16 + (j & 1) * 8;
+#pragma unroll
+    for (int i = 0; i < NA; i++) *reinterpret_cast<uint2 *>(dst + i * 1024) = dg[i];
+    r = mm_wave(r);
+    if ((tid & 63) == 0) red[tid >> 6] = r;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int w = 1; w < 4; w++) { mm_update(r, red[w].lo); mm_update(r, red[w].hi); }
+        const long b = ((long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        mm[2 * b] = (unsigned long long)r.lo ^ kSignFlip;
+        mm[2 * b + 1] = (unsigned long long)r.hi ^ kSignFlip;
+    }
+}
+
+// Folds the per-workgroup ranges of the pre-pass into range[0..1].
+__global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long long *mm, long count, unsigned long long *range)
+{
+    __shared__ unsigned long long lo_s[256], hi_s[256];
+    unsigned long long lo = ~0ull, hi = 0ull;
+    for (long i = threadIdx.x; i < count; i += 256) {
+        lo = mm[2 * i] < lo ? mm[2 * i] : lo;
+        hi = mm[2 * i + 1] > hi ? mm[2 * i + 1] : hi;
+    }
+    lo_s[threadIdx.x] = lo;
+    hi_s[threadIdx.x] = hi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 256; i++) { lo = lo_s[i] < lo ? lo_s[i] : lo; hi = hi_s[i] > hi ? hi_s[i] : hi; }
+        range[0] = lo;
+        range[1] = hi;
+    }
+}
+
+// ---- the GEMM kernel -------------------------------------------------------------------------------
+// WVM x WVN waves per workgroup, WM x WN 32x32 MFMA tiles per wave, KK MFMA k-depths (32 k each) per pipeline
+// step.  APL: A comes from pre-split digit planes (plain copy into LDS); otherwise it is split on the fly like B.
+//
+// The hot loop is branch-free: rows past M or N are clamped to the last valid row (their products land in
+// outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
+// own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
+// to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL>
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
+{
+    constexpr int T = 64 * WVM * WVN;
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 32 * KK, OCTS = BK / 8;
+    constexpr int RUN = B32 ? 4 : 2;
     constexpr int D = (NA + NB - 1) > 16 ? 16 : (NA + NB - 1);     // diagonal 16 has weight 2^128: dropped
     constexpr int A_BLOCKS = (BM / 32) * NA, B_BLOCKS = (BN / 32) * NB;
-    constexpr int STAGE = (A_BLOCKS + B_BLOCKS) * 1024;
+    constexpr int SUBSTAGE = (A_BLOCKS + B_BLOCKS) * 1024;
+    constexpr int STAGE = KK * SUBSTAGE;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WVN, wn = wave % WVN;
 
     // workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of them, each with its own L2), so
     // ids are regrouped to give each XCD a contiguous run of tiles; within a run the tile-row index moves
     // fastest, so the workgroups that share a B tile sit on the same L2.
-    int bid = blockIdx.x;
     const int per_batch = p.tiles_m * p.tiles_n;
     const int total = per_batch * gridDim.y;
-    int lin = blockIdx.y * per_batch + bid;
+    int lin = blockIdx.y * per_batch + blockIdx.x;
     if ((total & 7) == 0) lin = (lin & 7) * (total >> 3) + (lin >> 3);
     const int g = lin / per_batch;
     const int rem = lin - g * per_batch;
     const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int64_t *Ag = p.A + (long)g * p.sA;
-    const long boff = (long)g * p.sB;
-    const bool verify_a = tn == 0;
+    const bool verify_a = !APL && tn == 0;
     const bool verify_b = tm == 0 && (g == 0 || p.verify_b_all_batches);
     MinMax ra = { INT64_MAX, INT64_MIN }, rb = { INT64_MAX, INT64_MIN };
 
@@ -202,112 +353,169 @@ __global__ __launch_bounds__(256, 1) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[a][b][d][r] = 0;
 
-    // staging registers for the next k-step
-    constexpr int A_IT = BM / 64, B_IT = BN / 64;
+    // Work items of the loaders: (row, j) pairs owning 8 elements each, or 16-byte chunks of digit planes.
+    constexpr int A_ITEMS = BM * OCTS, B_ITEMS = BN * OCTS;
+    constexpr int A_IT = APL ? 1 : (A_ITEMS + T - 1) / T, B_IT = (B_ITEMS + T - 1) / T;
+    constexpr int A_CHUNKS = KK * A_BLOCKS * 64, A_CIT = APL ? (A_CHUNKS + T - 1) / T : 1;
     int64_t sa[A_IT][8], sb[B_IT][8];
+    v4i pa[A_CIT];
 
-    // loader coordinates.  k-contiguous operands: 4 threads cover the 32 k of one row.  k-major B: 64 consecutive
-    // threads cover 64 consecutive n of one k-octet.
-    const int a_row = tid >> 2, a_oct = tid & 3;
-    const int b_row = BKM ? (tid & 63) : (tid >> 2), b_oct = BKM ? (tid >> 6) : (tid & 3);
     const bool a_vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
     const bool b_vec = !BKM && (((uintptr_t)p.B | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
 
-    auto fetch = [&](int k0) {
+    // per-thread source pointers (advanced by BK per step) and LDS destinations
+    const int64_t *a_src[A_IT];
+    const unsigned char *a_pl[A_CIT];
+    const char *b_src[B_IT];
+    // LDS destinations are stage-relative; threads with no work in an iteration aim at a dummy area behind the two
+    // stages (and a zero stage stride), which keeps the loop body free of branches.
+    constexpr int DUMMY = 2 * STAGE;
+    int a_j[A_IT], b_j[B_IT], a_dst[A_IT], b_dst[B_IT], pl_dst[A_CIT];
+    int a_stride[A_IT], b_stride[B_IT], pl_stride[A_CIT];
+    if (APL) {
+#pragma unroll
+        for (int it = 0; it < A_CIT; it++) {
+            const int c = it * T + tid;
+            const bool live = A_CHUNKS % T == 0 || c < A_CHUNKS;
+            const int cc0 = live ? c : 0;
+            // LDS order inside a stage is [kk][sub][digit]; planes are [sub][ks32][digit]
+            const int kk = cc0 / (A_BLOCKS * 64), cc = cc0 - kk * (A_BLOCKS * 64);
+            const int sub_i = cc / (NA * 64), within = cc - sub_i * (NA * 64);
+            a_pl[it] = p.a_planes + (((long)g * p.a_msub + (m0 >> 5) + sub_i) * p.a_ksteps + kk) * (NA * 1024) + within * 16;
+            pl_dst[it] = live ? kk * SUBSTAGE + cc * 16 : DUMMY;
+            pl_stride[it] = live ? STAGE : 0;
+        }
+    } else {
 #pragma unroll
         for (int it = 0; it < A_IT; it++) {
-            const int m = m0 + it * 64 + a_row, k = k0 + a_oct * 8;
-            const int64_t *src = Ag + (long)m * p.lda + k;
-            if (m < p.M && k + 8 <= p.K && a_vec) {
+            const int idx = it * T + tid;
+            const bool live = A_ITEMS % T == 0 || idx < A_ITEMS;
+            const int row = (live ? idx : 0) / OCTS;
+            a_j[it] = idx % OCTS;
+            int m = m0 + row;
+            m = m < p.M ? m : p.M - 1;
+            a_src[it] = p.A + (long)g * p.sA + (long)m * p.lda;
+            a_dst[it] = live ? frag_offset(row, a_j[it], NA, SUBSTAGE) : DUMMY;
+            a_stride[it] = live ? STAGE : 0;
+        }
+    }
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const v4i t = reinterpret_cast<const v4i *>(src)[q];
-                    sa[it][2 * q] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
-                    sa[it][2 * q + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
-                }
-            } else {
+    for (int it = 0; it < B_IT; it++) {
+        const int idx = it * T + tid;
+        const bool live = B_ITEMS % T == 0 || idx < B_ITEMS;
+        const int idx0 = live ? idx : 0;
+        int row;
+        if (BKM) { row = (idx0 & 63) + 64 * (idx0 / (64 * OCTS)); b_j[it] = (idx0 >> 6) % OCTS; }
+        else { row = idx0 / OCTS; b_j[it] = idx0 % OCTS; }
+        int n = n0 + row;
+        n = n < p.N ? n : p.N - 1;
+        const long off = (long)g * p.sB + (long)n * p.ldbn;
+        b_src[it] = reinterpret_cast<const char *>(p.B) + off * (B32 ? 4 : 8);
+        b_dst[it] = live ? A_BLOCKS * 1024 + frag_offset(row, b_j[it], NB, SUBSTAGE) : DUMMY;
+        b_stride[it] = live ? STAGE : 0;
+    }
+
+    // L2 warm-up: one dword from every 64-byte line of the B tile ZK_PREFETCH steps ahead.  The value only feeds a
+    // store that never happens; issuing the loads after the real ones keeps them out of the real loads' waits.
+    constexpr int B_LINE_BYTES = BN * BK * (B32 ? 4 : 8);
+    constexpr int PF_IT = BKM ? 0 : (B_LINE_BYTES / 64 + T - 1) / T;
+    constexpr int LINES_PER_ROW = BK * (B32 ? 4 : 8) / 64;
+    const char *pf_src[PF_IT > 0 ? PF_IT : 1];
+    int pf_acc = 0;
 #pragma unroll
-                for (int q = 0; q < 8; q++) sa[it][q] = (m < p.M && k + q < p.K) ? src[q] : 0;
+    for (int it = 0; it < PF_IT; it++) {
+        const int l = it * T + tid;
+        int n = n0 + (l / LINES_PER_ROW) % BN;
+        n = n < p.N ? n : p.N - 1;
+        pf_src[it] = reinterpret_cast<const char *>(p.B) + ((long)g * p.sB + (long)n * p.ldbn) * (B32 ? 4 : 8) +
+                     (l % LINES_PER_ROW) * 64;
+    }
+    auto prefetch = [&](int ks) {
+#pragma unroll
+        for (int it = 0; it < PF_IT; it++)
+            pf_acc |= *reinterpret_cast<const int *>(pf_src[it] + (long)ks * BK * (B32 ? 4 : 8));
+    };
+
+    // FAST: the whole step lies inside K and the pointers allow 16-byte loads: no guards at all.
+    auto fetch = [&](int ks, auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+#ifdef ZK_DBG_SAME_TILE
+        ks = FAST ? (ks & 1) : ks;
+#endif
+        const int k0 = ks * BK;
+        if (APL) {
+#pragma unroll
+            for (int it = 0; it < A_CIT; it++)
+                pa[it] = *reinterpret_cast<const v4i *>(a_pl[it] + (long)ks * (KK * NA * 1024));
+        } else {
+#pragma unroll
+            for (int it = 0; it < A_IT; it++) {
+                if (FAST) load_owned_i64<RUN, OCTS>(a_src[it] + k0, a_j[it], true, BK, true, sa[it]);
+                else load_owned_i64<RUN, OCTS>(a_src[it] + k0, a_j[it], true, p.K - k0, false, sa[it]);
             }
         }
 #pragma unroll
         for (int it = 0; it < B_IT; it++) {
-            const int n = n0 + it * 64 + b_row, k = k0 + b_oct * 8;
             if (BKM) {
 #pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    const long off = boff + n + (long)(k + q) * p.ldbk;
+                for (int e = 0; e < 8; e++) {
+                    const int k = k0 + owned_k<RUN, OCTS>(b_j[it], e);
+                    const long off = (long)k * p.ldbk;
                     int64_t v = 0;
-                    if (n < p.N && k + q < p.K)
-                        v = B32 ? (int64_t)reinterpret_cast<const int32_t *>(p.B)[off]
-                                : reinterpret_cast<const int64_t *>(p.B)[off];
-                    sb[it][q] = v;
+                    if (FAST || k < p.K)
+                        v = B32 ? (int64_t)reinterpret_cast<const int32_t *>(b_src[it])[off]
+                                : reinterpret_cast<const int64_t *>(b_src[it])[off];
+                    sb[it][e] = v;
                 }
             } else if (B32) {
-                const int32_t *src = reinterpret_cast<const int32_t *>(p.B) + boff + (long)n * p.ldbn + k;
-                if (n < p.N && k + 8 <= p.K && b_vec) {
-#pragma unroll
-                    for (int q = 0; q < 2; q++) {
-                        const v4i t = reinterpret_cast<const v4i *>(src)[q];
-#pragma unroll
-                        for (int z = 0; z < 4; z++) sb[it][4 * q + z] = (int64_t)t[z];
-                    }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 8; q++) sb[it][q] = (n < p.N && k + q < p.K) ? (int64_t)src[q] : 0;
-                }
+                const int32_t *src = reinterpret_cast<const int32_t *>(b_src[it]) + k0;
+                if (FAST) load_owned_i32<RUN, OCTS>(src, b_j[it], true, BK, true, sb[it]);
+                else load_owned_i32<RUN, OCTS>(src, b_j[it], true, p.K - k0, false, sb[it]);
             } else {
-                const int64_t *src = reinterpret_cast<const int64_t *>(p.B) + boff + (long)n * p.ldbn + k;
-                if (n < p.N && k + 8 <= p.K && b_vec) {
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const v4i t = reinterpret_cast<const v4i *>(src)[q];
-                        sb[it][2 * q] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
-                        sb[it][2 * q + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
-                    }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 8; q++) sb[it][q] = (n < p.N && k + q < p.K) ? src[q] : 0;
-                }
+                const int64_t *src = reinterpret_cast<const int64_t *>(b_src[it]) + k0;
+                if (FAST) load_owned_i64<RUN, OCTS>(src, b_j[it], true, BK, true, sb[it]);
+                else load_owned_i64<RUN, OCTS>(src, b_j[it], true, p.K - k0, false, sb[it]);
             }
         }
     };
 
-    // digits of the staged rows -> LDS stage `buf`, fragment order
-    auto stash = [&](int buf) {
-        unsigned char *base = smem + buf * STAGE;
+    // staged elements -> digits -> LDS stage `buf`, fragment order
+    auto stash = [&](int buf, auto verify_tag) {
+        constexpr bool VERIFY = decltype(verify_tag)::value;
+        if (APL) {
 #pragma unroll
-        for (int it = 0; it < A_IT; it++) {
-            if (verify_a) {
+            for (int it = 0; it < A_CIT; it++)
+                *reinterpret_cast<v4i *>(smem + pl_dst[it] + buf * pl_stride[it]) = pa[it];
+        } else {
 #pragma unroll
-                for (int q = 0; q < 8; q++) mm_update(ra, sa[it][q]);
+            for (int it = 0; it < A_IT; it++) {
+                if (VERIFY && verify_a) {
+#pragma unroll
+                    for (int q = 0; q < 8; q++) mm_update(ra, sa[it][q]);
+                }
+                uint2 dg[NA];
+                limb_split8<NA>(sa[it], dg);
+#pragma unroll
+                for (int i = 0; i < NA; i++)
+                    *reinterpret_cast<uint2 *>(smem + a_dst[it] + buf * a_stride[it] + i * 1024) = dg[i];
             }
-            uint2 dg[NA];
-            limb_split8<NA>(sa[it], dg);
-            const int row = it * 64 + a_row;
-            const int slot = (row & 31) + 32 * (a_oct >> 1);
-            unsigned char *dst = base + ((row >> 5) * NA) * 1024 + slot * 16 + (a_oct & 1) * 8;
-#pragma unroll
-            for (int i = 0; i < NA; i++) *reinterpret_cast<uint2 *>(dst + i * 1024) = dg[i];
         }
 #pragma unroll
         for (int it = 0; it < B_IT; it++) {
-            if (verify_b) {
+            if (VERIFY && verify_b) {
 #pragma unroll
                 for (int q = 0; q < 8; q++) mm_update(rb, sb[it][q]);
             }
             uint2 dg[NB];
             limb_split8<NB>(sb[it], dg);
-            const int row = it * 64 + b_row;
-            const int slot = (row & 31) + 32 * (b_oct >> 1);
-            unsigned char *dst = base + (A_BLOCKS + (row >> 5) * NB) * 1024 + slot * 16 + (b_oct & 1) * 8;
 #pragma unroll
-            for (int i = 0; i < NB; i++) *reinterpret_cast<uint2 *>(dst + i * 1024) = dg[i];
+            for (int i = 0; i < NB; i++)
+                *reinterpret_cast<uint2 *>(smem + b_dst[it] + buf * b_stride[it] + i * 1024) = dg[i];
         }
     };
 
-    auto compute = [&](int buf) {
-        const unsigned char *base = smem + buf * STAGE;
+    auto compute = [&](int buf, int kk) {
+        const unsigned char *base = smem + buf * STAGE + kk * SUBSTAGE;
         v4i fa[WM][NA], fb[WN][NB];
 #pragma unroll
         for (int a = 0; a < WM; a++)
@@ -332,20 +540,50 @@ __global__ __launch_bounds__(256, 1) void gemm_mfma_kernel(MfmaParams p)
                 }
     };
 
-    const int ksteps = (p.K + 31) / 32;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int ks = 0; ks < ksteps; ks++) {
+    const int ksteps = (p.K + BK - 1) / BK;
+    const int full_steps = (a_vec || APL) && (b_vec || BKM) ? p.K / BK : 0;     // steps that can use unguarded loads
+
+    auto step_body = [&](int ks, auto fast_tag, auto verify_tag) {
         const int cur = ks & 1;
-        if (ks + 1 < ksteps) fetch((ks + 1) * 32);
-        compute(cur);
-        if (ks + 1 < ksteps) stash(cur ^ 1);
+        fetch(ks + 1, fast_tag);
+        if (decltype(fast_tag)::value && ZK_PREFETCH > 0 && ks + 1 + ZK_PREFETCH < full_steps) prefetch(ks + 1 + ZK_PREFETCH);
+#pragma unroll
+        for (int kk = 0; kk < KK - 1; kk++) compute(cur, kk);
+        if (KK > 1) __builtin_amdgcn_sched_barrier(0);
+        compute(cur, KK - 1);
+        stash(cur ^ 1, verify_tag);
+        if (decltype(fast_tag)::value && !decltype(verify_tag)::value) {
+            constexpr int MFMAS = WM * WN * NA * NB;
+#pragma unroll
+            for (int i = 0; i < MFMAS; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, ZK_VALU_PER_MFMA, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+        }
         __syncthreads();
+    };
+
+    if (full_steps > 0) fetch(0, std::true_type()); else fetch(0, std::false_type());
+    stash(0, std::true_type());
+    __syncthreads();
+    int ks = 0;
+    if (verify_a || verify_b) {
+        for (; ks + 1 < full_steps; ks++) step_body(ks, std::true_type(), std::true_type());
+    } else {
+        for (; ks + 1 < full_steps; ks++) step_body(ks, std::true_type(), std::false_type());
+    }
+    for (; ks + 1 < ksteps; ks++) step_body(ks, std::false_type(), std::true_type());
+    {
+        const int cur = (ksteps - 1) & 1;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) compute(cur, kk);
     }
 
     if (verify_a) mm_publish(ra, p.range);
     if (verify_b) mm_publish(rb, p.range + 2);
+    if (pf_acc == 0x7f3a91c5 && p.shift == 99) p.C[0] = pf_acc;      // never true: keeps the warm-up loads alive
 
     // epilogue: diagonals -> 128-bit sum -> shift.  Accumulator register r of lane l holds
     // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile.
@@ -386,24 +624,40 @@ __global__ __launch_bounds__(256, 1) void gemm_mfma_kernel(MfmaParams p)
 
 // ---- host side ---------------------------------------------------------------------------------------
 typedef void (*MfmaKernel)(MfmaParams);
+typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
+
+enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kVariants };
 
 struct Instance {
-    int na, nb, wm, wn;
-    MfmaKernel fn[2][2];     // [b32][kmajor]
+    int na, nb, bm, bn, threads, kk;
+    MfmaKernel fn[kVariants];
+    PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
 };
 
-template <int NA, int NB, int WM, int WN>
+
+template <int NA, int NB>
 static Instance make_instance()
 {
+    constexpr int DD = NA + NB - 1;
+    // narrow: 8 waves as 2x4, 64x32 per wave (128x128); mid: 8 waves as 4x2, 32x32 per wave (128x64);
+    // wide: 4 waves as 2x2, 32x32 per wave (64x64, one wave per SIMD because of the accumulator count)
+    constexpr int WVM = DD <= 5 ? 2 : (DD <= 10 ? 4 : 2);
+    constexpr int WVN = DD <= 5 ? 4 : 2;
+    constexpr int WM = DD <= 5 ? 2 : 1, WN = 1;
+    constexpr int KK = ZK_KK(DD);
     Instance s;
-    s.na = NA; s.nb = NB; s.wm = WM; s.wn = WN;
-    s.fn[0][0] = gemm_mfma_kernel<NA, NB, WM, WN, false, false>;
-    s.fn[0][1] = gemm_mfma_kernel<NA, NB, WM, WN, false, true>;
-    s.fn[1][0] = s.fn[1][1] = nullptr;
+    s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
+    for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
+    s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false>;
+    s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true>;
+    s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false>;
     if constexpr (NB <= 5) {          // int32 values never need more than five digits
-        s.fn[1][0] = gemm_mfma_kernel<NA, NB, WM, WN, true, false>;
-        s.fn[1][1] = gemm_mfma_kernel<NA, NB, WM, WN, true, true>;
+        s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false>;
+        s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true>;
+        s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false>;
     }
+    s.planes[0] = a_planes_kernel<NA, 2, KK>;
+    s.planes[1] = a_planes_kernel<NA, 4, KK>;
     return s;
 }
 
@@ -411,10 +665,13 @@ static Instance make_instance()
 static const Instance *instances(int *count)
 {
     static const Instance table[] = {
-        make_instance<3, 3, 2, 2>(), make_instance<4, 3, 2, 1>(), make_instance<4, 4, 2, 1>(),
-        make_instance<5, 4, 2, 1>(), make_instance<5, 5, 2, 1>(), make_instance<6, 5, 2, 1>(),
-        make_instance<3, 5, 2, 1>(), make_instance<6, 3, 2, 1>(),
-        make_instance<9, 5, 1, 1>(), make_instance<5, 9, 1, 1>(), make_instance<9, 9, 1, 1>(),
+#ifdef ZK_PROBE
+        ZK_PROBE
+#else
+        make_instance<3, 3>(), make_instance<4, 3>(), make_instance<4, 4>(), make_instance<5, 4>(),
+        make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(),
+        make_instance<9, 5>(), make_instance<5, 9>(), make_instance<9, 9>(),
+#endif
     };
     *count = (int)(sizeof(table) / sizeof(table[0]));
     return table;
@@ -428,9 +685,8 @@ static const Instance *pick_instance(int na, int nb, bool b32)
     long best_cost = 0;
     for (int i = 0; i < count; i++) {
         if (t[i].na < na || t[i].nb < nb) continue;
-        if (b32 && !t[i].fn[1][0]) continue;
-        // MFMA work per output tile area, penalised a little for the smaller wave tiles
-        long cost = (long)t[i].na * t[i].nb * 8 + (4 - t[i].wm * t[i].wn);
+        if (b32 && !t[i].fn[kB32Fly]) continue;
+        long cost = (long)t[i].na * t[i].nb;
         if (!best || cost < best_cost) { best = &t[i]; best_cost = cost; }
     }
     return best;
@@ -439,7 +695,11 @@ static const Instance *pick_instance(int na, int nb, bool b32)
 struct RangeCache {
     std::mutex mu;
     std::map<std::tuple<const void *, long, long, int>, int> limbs;     // (ptr, rows, K, elem size) -> digits
-    unsigned long long *dev = nullptr;
+    unsigned long long *dev = nullptr;       // [minA, maxA, minB, maxB]
+    unsigned char *planes = nullptr;         // digit planes of A, grown on demand, kept for the process lifetime
+    size_t planes_bytes = 0;
+    unsigned long long *mm = nullptr;        // per-workgroup ranges of the plane pre-pass
+    size_t mm_count = 0;
     int lookup(const void *ptr, long rows, long K, int esz)
     {
         auto it = limbs.find(std::make_tuple(ptr, rows, K, esz));
@@ -482,6 +742,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift; p.init = d.init;
     p.range = g_cache.dev;
     p.verify_b_all_batches = d.sB != 0;
+    p.a_planes = nullptr; p.a_msub = 0; p.a_ksteps = 0;
+    p.dbg = 0;
 
     const long rows_a = (long)d.G * d.M;
     int na = g_cache.lookup(d.A, rows_a, d.K, 8);
@@ -501,15 +763,57 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (!inst) return false;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
-        const long kpad = ((long)d.K + 31) / 32 * 32;
-        if (pairs * kpad * 16384 > 0x7FFFFFFFL) return false;
-        MfmaKernel fn = inst->fn[d.b32 ? 1 : 0][kmajor ? 1 : 0];
-        const int BM = 64 * inst->wm, BN = 64 * inst->wn;
+        const int ksteps = ((d.K + 32 * inst->kk - 1) / (32 * inst->kk)) * inst->kk;     // 32-k steps, padded
+        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return false;
+        const int BM = inst->bm, BN = inst->bn;
         p.tiles_m = (d.M + BM - 1) / BM;
         p.tiles_n = (d.N + BN - 1) / BN;
         const long per_batch = (long)p.tiles_m * p.tiles_n;
         if (per_batch > 0x7FFFFFFFL) return false;
-        const size_t lds = 2 * (size_t)((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024;
+        // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass
+        const bool use_planes = !kmajor && p.tiles_n >= 4;
+        const int variant = kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
+                                   : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
+        MfmaKernel fn = inst->fn[variant];
+        if (!fn) return false;
+        range_reset_kernel<<<1, 64, 0, 0>>>(p.range);
+        if (use_planes) {
+            const int msub = p.tiles_m * (BM / 32);
+            const size_t need = (size_t)d.G * msub * ksteps * inst->na * 1024;
+            if (need > g_cache.planes_bytes) {
+                if (g_cache.planes && hipFree(g_cache.planes) != hipSuccess) {
+                    set_error(kLaunchFailure, "gemm: cannot release the digit-plane buffer");
+                    return false;
+                }
+                g_cache.planes = nullptr;
+                g_cache.planes_bytes = 0;
+                if (hipMalloc(&g_cache.planes, need) != hipSuccess) {
+                    (void)hipGetLastError();
+                    return false;                    // not enough memory for planes: the caller uses the VALU path
+                }
+                g_cache.planes_bytes = need;
+            }
+            p.a_planes = g_cache.planes; p.a_msub = msub; p.a_ksteps = ksteps;
+            const int rows_per_wg = 256 / (4 * inst->kk);
+            const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)(msub * 32 / rows_per_wg), (unsigned)d.G);
+            const size_t wgs = (size_t)pgrid.x * pgrid.y * pgrid.z;
+            if (wgs > g_cache.mm_count) {
+                if (g_cache.mm && hipFree(g_cache.mm) != hipSuccess) {
+                    set_error(kLaunchFailure, "gemm: cannot release the range scratch");
+                    return false;
+                }
+                g_cache.mm = nullptr;
+                g_cache.mm_count = 0;
+                if (hipMalloc(&g_cache.mm, wgs * 2 * sizeof(unsigned long long)) != hipSuccess) {
+                    (void)hipGetLastError();
+                    return false;
+                }
+                g_cache.mm_count = wgs;
+            }
+            inst->planes[d.b32 ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
+            range_fold_kernel<<<1, 256, 0, 0>>>(g_cache.mm, (long)wgs, p.range);
+        }
+        const size_t lds = 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
         static std::set<const void *> lds_raised;
         if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
             if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
@@ -518,8 +822,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             }
             lds_raised.insert((const void *)fn);
         }
-        range_reset_kernel<<<1, 64, 0, 0>>>(p.range);
-        fn<<<dim3((unsigned)per_batch, (unsigned)d.G), dim3(256), lds, 0>>>(p);
+        fn<<<dim3((unsigned)per_batch, (unsigned)d.G), dim3((unsigned)inst->threads), lds, 0>>>(p);
         if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
