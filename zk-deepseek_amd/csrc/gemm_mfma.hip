@@ -339,8 +339,12 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const bool verify_a = !APL && tn == 0;
-    const bool verify_b = tm == 0 && (g == 0 || p.verify_b_all_batches);
+    // Range tracking is shared out: the tiles_m workgroups that load the same B tile each check every
+    // tiles_m-th k-step of it (likewise for A across the workgroups of a tile row), so no workgroup is slower
+    // than its neighbours and every element is still seen once.
+    const int vmod_b = p.tiles_m < 8 ? p.tiles_m : 8, vmod_a = p.tiles_n < 8 ? p.tiles_n : 8;
+    const bool verify_a = !APL && tn < vmod_a;
+    const bool verify_b = tm < vmod_b && (g == 0 || p.verify_b_all_batches);
     MinMax ra = { INT64_MAX, INT64_MIN }, rb = { INT64_MAX, INT64_MIN };
 
     v16i acc[WM][WN][D];
@@ -415,13 +419,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         b_stride[it] = live ? STAGE : 0;
     }
 
-    // L2 warm-up: one dword from every 64-byte line of the B tile ZK_PREFETCH steps ahead.  The value only feeds a
-    // store that never happens; issuing the loads after the real ones keeps them out of the real loads' waits.
-    constexpr int B_LINE_BYTES = BN * BK * (B32 ? 4 : 8);
-    constexpr int PF_IT = BKM ? 0 : (B_LINE_BYTES / 64 + T - 1) / T;
-    constexpr int LINES_PER_ROW = BK * (B32 ? 4 : 8) / 64;
+    // L2 warm-up: one dword from every 64-byte line of the B tile ZK_PREFETCH steps ahead of the staged loads.  The
+    // value only feeds a store that never happens; being issued after the real loads, it never delays their wait.
+    constexpr int B_STEP_BYTES = BK * (B32 ? 4 : 8);
+    constexpr int LINES_PER_ROW = B_STEP_BYTES / 64 > 0 ? B_STEP_BYTES / 64 : 1;
+    constexpr int PF_IT = (BKM || ZK_PREFETCH == 0) ? 0 : (BN * LINES_PER_ROW + T - 1) / T;
     const char *pf_src[PF_IT > 0 ? PF_IT : 1];
-    int pf_acc = 0;
+    int pf_acc = 0, pf_val[PF_IT > 0 ? PF_IT : 1] = { 0 };
 #pragma unroll
     for (int it = 0; it < PF_IT; it++) {
         const int l = it * T + tid;
@@ -432,8 +436,10 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     }
     auto prefetch = [&](int ks) {
 #pragma unroll
-        for (int it = 0; it < PF_IT; it++)
-            pf_acc |= *reinterpret_cast<const int *>(pf_src[it] + (long)ks * BK * (B32 ? 4 : 8));
+        for (int it = 0; it < PF_IT; it++) {
+            pf_acc |= pf_val[it];          // the value loaded one step ago: long since landed, no wait
+            pf_val[it] = *reinterpret_cast<const int *>(pf_src[it] + (long)ks * B_STEP_BYTES);
+        }
     };
 
     // FAST: the whole step lies inside K and the pointers allow 16-byte loads: no guards at all.
@@ -480,8 +486,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     };
 
     // staged elements -> digits -> LDS stage `buf`, fragment order
-    auto stash = [&](int buf, auto verify_tag) {
-        constexpr bool VERIFY = decltype(verify_tag)::value;
+    auto stash = [&](int buf) {
         if (APL) {
 #pragma unroll
             for (int it = 0; it < A_CIT; it++)
@@ -489,10 +494,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         } else {
 #pragma unroll
             for (int it = 0; it < A_IT; it++) {
-                if (VERIFY && verify_a) {
-#pragma unroll
-                    for (int q = 0; q < 8; q++) mm_update(ra, sa[it][q]);
-                }
                 uint2 dg[NA];
                 limb_split8<NA>(sa[it], dg);
 #pragma unroll
@@ -502,10 +503,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         }
 #pragma unroll
         for (int it = 0; it < B_IT; it++) {
-            if (VERIFY && verify_b) {
-#pragma unroll
-                for (int q = 0; q < 8; q++) mm_update(rb, sb[it][q]);
-            }
             uint2 dg[NB];
             limb_split8<NB>(sb[it], dg);
 #pragma unroll
@@ -514,9 +511,9 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         }
     };
 
-    auto compute = [&](int buf, int kk) {
+    // Fragments of one MFMA depth, and the MFMAs of a slice [LO, HI) of the depth's (i, j, tile) list.
+    auto load_frags = [&](int buf, int kk, v4i (&fa)[WM][NA], v4i (&fb)[WN][NB]) {
         const unsigned char *base = smem + buf * STAGE + kk * SUBSTAGE;
-        v4i fa[WM][NA], fb[WN][NB];
 #pragma unroll
         for (int a = 0; a < WM; a++)
 #pragma unroll
@@ -527,59 +524,96 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
             for (int j = 0; j < NB; j++)
                 fb[b][j] = *reinterpret_cast<const v4i *>(base + ((A_BLOCKS + (wn * WN + b) * NB + j) * 1024) + lane * 16);
+    };
+    constexpr int MFMAS = WM * WN * NA * NB;
+    auto mfma_slice = [&](auto lo_tag, auto hi_tag, const v4i (&fa)[WM][NA], const v4i (&fb)[WN][NB]) {
+        constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
 #pragma unroll
         for (int i = 0; i < NA; i++)
 #pragma unroll
             for (int j = 0; j < NB; j++)
-                if (i + j < D) {
 #pragma unroll
-                    for (int a = 0; a < WM; a++)
+                for (int a = 0; a < WM; a++)
 #pragma unroll
-                        for (int b = 0; b < WN; b++)
+                    for (int b = 0; b < WN; b++) {
+                        const int idx = ((i * NB + j) * WM + a) * WN + b;
+                        if (idx >= LO && idx < HI && i + j < D)
                             acc[a][b][i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a][i], fb[b][j], acc[a][b][i + j], 0, 0, 0);
-                }
+                    }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, MFMAS / 2> IH;
+    typedef std::integral_constant<int, MFMAS> IF;
+    auto compute_all = [&](int buf) {
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+            v4i fa[WM][NA], fb[WN][NB];
+            load_frags(buf, kk, fa, fb);
+            mfma_slice(I0(), IF(), fa, fb);
+        }
     };
 
     const int ksteps = (p.K + BK - 1) / BK;
     const int full_steps = (a_vec || APL) && (b_vec || BKM) ? p.K / BK : 0;     // steps that can use unguarded loads
 
-    auto step_body = [&](int ks, auto fast_tag, auto verify_tag) {
-        const int cur = ks & 1;
-        fetch(ks + 1, fast_tag);
-        if (decltype(fast_tag)::value && ZK_PREFETCH > 0 && ks + 1 + ZK_PREFETCH < full_steps) prefetch(ks + 1 + ZK_PREFETCH);
+    // Range tracking of the staged elements of data step d, done while the registers still hold them.
+    auto track = [&](int d) {
+        if (verify_a && d % vmod_a == tn) {
 #pragma unroll
-        for (int kk = 0; kk < KK - 1; kk++) compute(cur, kk);
-        if (KK > 1) __builtin_amdgcn_sched_barrier(0);
-        compute(cur, KK - 1);
-        stash(cur ^ 1, verify_tag);
-        if (decltype(fast_tag)::value && !decltype(verify_tag)::value) {
-            constexpr int MFMAS = WM * WN * NA * NB;
+            for (int it = 0; it < A_IT; it++)
 #pragma unroll
-            for (int i = 0; i < MFMAS; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, ZK_VALU_PER_MFMA, 0);
-                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            }
+                for (int q = 0; q < 8; q++) mm_update(ra, sa[it][q]);
         }
+        if (verify_b && d % vmod_b == tm) {
+#pragma unroll
+            for (int it = 0; it < B_IT; it++)
+#pragma unroll
+                for (int q = 0; q < 8; q++) mm_update(rb, sb[it][q]);
+        }
+    };
+
+    // One pipeline step, three fenced phases:
+    //   A  fragment reads of stage `cur` and the first half of its MFMAs (time for the staged loads to land);
+    //   B  the second half of the MFMAs interleaved, in one scheduling region, with the digit split of the
+    //      elements staged for step ks+1 and their LDS writes into the other stage;
+    //   C  the loads of step ks+2 into the now free staging registers, then the barrier.
+    auto step_body = [&](int ks, auto fast_tag) {
+        const int cur = ks & 1;
+#pragma unroll
+        for (int kk = 0; kk < KK - 1; kk++) {
+            v4i fa[WM][NA], fb[WN][NB];
+            load_frags(cur, kk, fa, fb);
+            mfma_slice(I0(), IF(), fa, fb);
+        }
+        v4i fa[WM][NA], fb[WN][NB];
+        load_frags(cur, KK - 1, fa, fb);
+        mfma_slice(I0(), IH(), fa, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_slice(IH(), IF(), fa, fb);
+        stash(cur ^ 1);
+#pragma unroll
+        for (int i = 0; i < MFMAS - MFMAS / 2; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, ZK_VALU_PER_MFMA, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        track(ks + 1);
+        if (ks + 2 < ksteps) fetch(ks + 2, fast_tag);
+        if (ZK_PREFETCH > 0 && decltype(fast_tag)::value && ks + 2 + ZK_PREFETCH < full_steps) prefetch(ks + 2 + ZK_PREFETCH);
         __syncthreads();
     };
 
+    // prologue: stage 0 holds step 0, the staging registers hold step 1
     if (full_steps > 0) fetch(0, std::true_type()); else fetch(0, std::false_type());
-    stash(0, std::true_type());
+    track(0);
+    stash(0);
+    if (ksteps > 1) { if (full_steps > 1) fetch(1, std::true_type()); else fetch(1, std::false_type()); }
     __syncthreads();
     int ks = 0;
-    if (verify_a || verify_b) {
-        for (; ks + 1 < full_steps; ks++) step_body(ks, std::true_type(), std::true_type());
-    } else {
-        for (; ks + 1 < full_steps; ks++) step_body(ks, std::true_type(), std::false_type());
-    }
-    for (; ks + 1 < ksteps; ks++) step_body(ks, std::false_type(), std::true_type());
-    {
-        const int cur = (ksteps - 1) & 1;
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++) compute(cur, kk);
-    }
+    for (; ks + 2 < full_steps; ks++) step_body(ks, std::true_type());
+    for (; ks + 1 < ksteps; ks++) step_body(ks, std::false_type());
+    compute_all((ksteps - 1) & 1);
 
     if (verify_a) mm_publish(ra, p.range);
     if (verify_b) mm_publish(rb, p.range + 2);
