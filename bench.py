@@ -30,7 +30,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,cpu,calib (default gemm,extra,cpu)")
     return ap.parse_args()
 
 
@@ -129,7 +129,7 @@ def main():
         ops = 2.0 * pairs * macs                         # i8 multiply-adds issued as MFMA, counted as 2 ops
         achieved = ops / (kern_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": I8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                    "frac": achieved / I8_MFMA_PEAK_TOPS, "traffic": None,
+                    "frac": achieved / I8_MFMA_PEAK_TOPS, "traffic": measured_traffic(),
                     "note": "i8 MFMA ops = 2 * limbs_a * limbs_b * M*N*K (%dx%d limb pairs per int64 MAC); "
                             "duration = HIP events over the whole launcher" % (la, lb)}
     else:
@@ -201,6 +201,16 @@ def main():
                 Ar.numel(), extra_bytes=4.0 * 7168 + 8.0 * Mr, steps=20)
             del Ar, Cr
 
+    if "calib" in legs:
+        # plain copy of known size (1 GiB in, 1 GiB out): what FETCH_SIZE / WRITE_SIZE read for it is the
+        # scale factor applied to the same counters of the GEMM kernel (see profiles/)
+        src = torch.empty((1 << 27,), dtype=torch.int64, device="cuda").fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     cpu_baseline = None
     if "cpu" in legs:
         cpu_baseline = cpu_leg(A_h, W_h, c)
@@ -219,6 +229,16 @@ def main():
         "extra": extra,
     }
     print(json.dumps(out))
+
+
+def measured_traffic():
+    """HBM bytes per launch of the config-4 GEMM kernel, from the committed rocprofv3 --pmc runs (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB copy): profiles/traffic.json."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get("gemm_config4_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
 
 
 def cpu_leg(A_h, W_h, c):
