@@ -1,0 +1,209 @@
+"""The layer arithmetic around the kernels, restated once and run on two back ends.
+
+The reference's `inference/model.py` glues the kernels together with plain int64 tensor ops (scale
+ladders, the SiLU gate product, softmax scale 94/695, the causal mask, gate routing, residual adds).
+This module restates that glue (file:line cited per function) over a tiny back-end interface so that the
+same code runs on the GPU (the `kernel` module + torch) and on the CPU oracle (+ numpy); the tests
+compare the two bit for bit.  Nothing here is product code.
+"""
+import numpy as np
+
+
+class CpuBackend:
+    """numpy arrays + the CPU oracle"""
+
+    def __init__(self, oracle):
+        self.o = oracle
+        self.lut19 = oracle.softmax_init_q19()
+        self.lut23 = oracle.silu_init_q23()
+
+    def linear(self, x, w, shift):
+        return self.o.int64_bmm_broadcast(x, w, 1, 1, shift)
+
+    def silu(self, x):
+        return self.o.silu_q23(x, self.lut23)
+
+    def sigmoid(self, x):
+        return self.o.sigmoid_q23(x, self.lut23)
+
+    def softmax(self, x):
+        return self.o.softmax_q19(x, self.lut19)[0]
+
+    def rmsnorm(self, x2d, w, dim):
+        return self.o.RMS_Norm_int64(x2d, w, 1, dim)[0]
+
+    def rope(self, x, table):
+        return self.o.complex_int64_mul_broadcast(x, table)
+
+    def einsum(self, name, a, b, shift):
+        return getattr(self.o, name)(np.ascontiguousarray(a), np.ascontiguousarray(b), shift)
+
+    def causal_mask(self, S, T):
+        return np.triu(np.full((S, T), -(64 << 36), np.int64), 1)
+
+    def to_host(self, x):
+        return np.asarray(x)
+
+    def from_host(self, x):
+        return np.ascontiguousarray(x)
+
+    def zeros_like(self, x):
+        return np.zeros_like(x)
+
+    def index_add_rows(self, y, idx, v):
+        np.add.at(y, idx, v)
+        return y
+
+
+class GpuBackend:
+    """torch CUDA tensors + the HIP library through `kernel`"""
+
+    def __init__(self, kernel):
+        import torch
+        self.t = torch
+        self.k = kernel
+        kernel.softmax_init_q19()
+        kernel.silu_init_q23()
+
+    def linear(self, x, w, shift):
+        return self.k.int64_bmm_broadcast(x.contiguous(), w, 1, 1, shift)
+
+    def silu(self, x):
+        out = self.t.empty_like(x)
+        self.k.silu_q23(x.contiguous(), out)
+        return out
+
+    def sigmoid(self, x):
+        out = self.t.empty_like(x)
+        self.k.sigmoid_q23(x.contiguous(), out)
+        return out
+
+    def softmax(self, x):
+        out = self.t.empty_like(x)
+        self.k.softmax_q19(x.contiguous(), out)
+        return out
+
+    def rmsnorm(self, x2d, w, dim):
+        return self.k.RMS_Norm_int64(x2d.contiguous(), w, 1, dim)[0]
+
+    def rope(self, x, table):
+        return self.k.complex_int64_mul_broadcast(x.contiguous(), table.contiguous())
+
+    def einsum(self, name, a, b, shift):
+        return getattr(self.k, name)(a.contiguous(), b.contiguous(), shift)
+
+    def causal_mask(self, S, T):
+        return self.t.full((S, T), -(64 << 36), dtype=self.t.int64, device="cuda").triu_(1)
+
+    def to_host(self, x):
+        return x.cpu().numpy()
+
+    def from_host(self, x):
+        return self.t.from_numpy(np.ascontiguousarray(x)).cuda()
+
+    def zeros_like(self, x):
+        return self.t.zeros_like(x)
+
+    def index_add_rows(self, y, idx, v):
+        y.index_add_(0, idx, v)
+        return y
+
+
+def expert_ffn(be, x, w1, w2, w3, c13, c2):
+    """gate/up GEMMs, SiLU gate, down GEMM: MLP_int.forward / Expert_int.forward
+    (inference/model.py:1018-1049, 1247-1281).  x [1,M,dim] Q23 activations."""
+    r1, _ = be.linear(x, w1, c13)
+    r2, _ = be.linear(x, w3, c13)
+    s1 = be.silu(r1)
+    h = (s1 * r2) >> 23                     # model.py:1048 uses // 2^23, :1280 uses >> 23: the same floor
+    y, _ = be.linear(h, w2, c2)
+    return y
+
+
+def attention_scores_softmax_pv(be, q_nope, q_pe, kv_cache, pe_cache, causal=True):
+    """scores = ((q_nope.kv + 11)>>23 + (q_pe.pe + 10)>>21) * 94 // 695 + mask; softmax_q19; P.V >> 23
+    (inference/model.py:884-936).  q_nope [1,S,H,C], q_pe [1,S,H,R], kv_cache [1,T,C], pe_cache [1,T,R]."""
+    s1 = be.einsum("einsum_bshc_btc_bsht", q_nope, kv_cache, 23)
+    s2 = be.einsum("einsum_bshc_btc_bsht", q_pe, pe_cache, 21)
+    scores = (s1 + s2) * 94 // 695           # floor division (model.py:897)
+    if causal:
+        S, T = scores.shape[1], scores.shape[3]
+        m = be.causal_mask(S, T)
+        scores = scores + m[:, None, :]      # mask.unsqueeze(1) (model.py:905)
+    p = be.softmax(scores)
+    out = be.einsum("einsum_bsht_btc_bshc", p, kv_cache, 23)
+    return scores, p, out
+
+
+def mla(be, x, P, freqs, cfg):
+    """MLA.forward in absorb mode at start_pos = 0 (inference/model.py:747-957).  x [1,S,dim]."""
+    S, H = x.shape[1], cfg["heads"]
+    q_down, _ = be.linear(x, P["wq_a"], 30)
+    q_normed = be.rmsnorm(q_down[0], P["q_norm"], cfg["q_lora"])[None]
+    q_nope, _ = be.linear(q_normed, P["wq_b1"], 30)
+    q_pe, _ = be.linear(q_normed, P["wq_b2"], 30)
+    q_nope = q_nope.reshape(1, S, H, cfg["nope"])
+    q_pe = q_pe.reshape(1, S, H, cfg["rope"] // 2, 2)
+    q_pe = be.rope(q_pe, freqs).reshape(1, S, H, cfg["rope"])
+    kv, _ = be.linear(x, P["wkv_a1"], 29)
+    k_pe, _ = be.linear(x, P["wkv_a2"], 29)
+    k_pe = be.rope(k_pe.reshape(1, S, 1, cfg["rope"] // 2, 2), freqs).reshape(1, S, cfg["rope"])
+    q_abs = be.einsum("einsum_bshd_hdc_bshc", q_nope, P["wkv_b_1"], cfg["wkv_b_1_scale"])
+    kv_normed = be.rmsnorm(kv[0], P["kv_norm"], cfg["kv_lora"])[None]
+    _, _, o = attention_scores_softmax_pv(be, q_abs, q_pe, kv_normed, k_pe)
+    o = be.einsum("einsum_bshc_hdc_bshd", o, P["wkv_b_2"], cfg["wkv_b_2_scale"])
+    y, _ = be.linear(o.reshape(1, S, H * cfg["v"]), P["wo"], cfg["wo_scale"])
+    return y
+
+
+def gate_scores(be, x, P, cfg):
+    """the kernel part of Gate.forward: linear at the gate's scale, then sigmoid_q23 (model.py:1116-1135)"""
+    s, _ = be.linear(x, P["gate"], cfg["gate_scale"])
+    return be.sigmoid(s)[0]
+
+
+def route(scores_host, bias, cfg):
+    """the tensor-op part of Gate.forward (model.py:1160-1208) on the host, with exact integers; returns
+    (weights [T,topk], indices [T,topk]).  Ties are broken by lowest index, as a stable sort does."""
+    T, E = scores_host.shape
+    orig = scores_host
+    sc = scores_host + bias[None, :]
+    g = cfg["groups"]
+    grp = sc.reshape(T, g, E // g)
+    top2 = -np.sort(-grp, axis=-1)[..., :2].sum(-1)
+    gsel = np.argsort(-top2, axis=-1, kind="stable")[:, :cfg["topk_groups"]]
+    keep = np.zeros((T, g), bool)
+    np.put_along_axis(keep, gsel, True, axis=1)
+    sc = np.where(np.repeat(keep, E // g, axis=1), sc, -(1 << 42))
+    idx = np.argsort(-sc, axis=-1, kind="stable")[:, :cfg["topk"]]
+    w = np.take_along_axis(orig, idx, axis=1)
+    w = (w * (1 << 23)) // w.sum(-1, keepdims=True)
+    w = w * 5 // 2
+    return w, idx
+
+
+def moe(be, x, P, cfg):
+    """MoE.forward (inference/model.py:1325-1383): shared expert + top-k routed experts, weights Q23"""
+    T = x.shape[1]
+    sc = gate_scores(be, x, P, cfg)
+    w_host, idx_host = route(be.to_host(sc), P["gate_bias_host"], cfg)
+    y = be.zeros_like(x[0])
+    for e in range(cfg["experts"]):
+        tok, slot = np.nonzero(idx_host == e)
+        if tok.size == 0:
+            continue
+        xe = x[0][be.from_host(tok)][None]
+        ye = expert_ffn(be, xe, P["w1"][e], P["w2"][e], P["w3"][e], cfg["c13"], cfg["c2"])[0]
+        we = be.from_host(w_host[tok, slot].astype(np.int64))[:, None]
+        y = be.index_add_rows(y, be.from_host(tok), (ye * we) // (1 << 23))      # model.py:1379
+    z = expert_ffn(be, x, P["sw1"], P["sw2"], P["sw3"], cfg["c13"], cfg["c2"])
+    return y[None] + z, idx_host
+
+
+def decoder_layer(be, x, P, freqs, cfg):
+    """Block.forward for a MoE layer (inference/model.py:1430-1475): x Q31 residual stream [1,S,dim]"""
+    a = be.rmsnorm(x[0], P["attn_norm"], cfg["dim"])[None]
+    x = x + mla(be, a, P, freqs, cfg) * (1 << 12)               # model.py:1465
+    f = be.rmsnorm(x[0], P["ffn_norm"], cfg["dim"])[None]
+    y, idx = moe(be, f, P, cfg)
+    return x + y * (1 << 8), idx                                 # model.py:1472
