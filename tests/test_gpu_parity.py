@@ -409,3 +409,30 @@ def test_gemm_mfma_path_is_taken(K, oracle):
     C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
     assert K.gemm_last_plan() == (1, 0, 0)
     K.lib.zk_gemm_set_path(0)
+
+
+@pytest.mark.parametrize("fn,Q", ACTS)
+def test_activation_table_path(K, oracle, fn, Q):
+    """tensors of 2^20 elements or more take the quotient-table kernel: in-range values, both saturation sides, the
+    shifts outside the table (|x| > 16.6), the overflowing-shift region, full-range garbage and a hostile table (which
+    must switch the kernel back to per-element division) all have to match the oracle"""
+    one = 1 << Q
+    rng = np.random.default_rng(100 + Q)
+    n = (1 << 20) + 3
+    x = rng.integers(-(18 << Q), 18 << Q, size=n, dtype=np.int64)
+    x[:4000] = rng.integers(-64 * one, 64 * one, size=4000, dtype=np.int64)
+    x[4000:8000] = rand_i64(rng, (4000,), 63)
+    x[8000:8016] = [0, 1, -1, 64 * one, 64 * one - 1, -64 * one, -64 * one + 1, 100 * one, -100 * one, -(1 << 63),
+                    (1 << 63) - 1, -28 * one, -44 * one, -45 * one, -63 * one, 17 * one]
+    x = x.reshape(1, 1, n)
+    oracle.set_threads(oracle.max_threads())
+    default = K.EXP2_FRAC_LUT_Q23 if Q == 23 else K.EXP2_FRAC_LUT_Q25
+    for table in (None, rand_i64(rng, (256,), 63), rng.integers(0, 1 << 40, size=256, dtype=np.int64)):
+        R = dev(x)
+        C = torch.empty_like(R)
+        t = default if table is None else dev(table)
+        getattr(K.lib, fn)(R.data_ptr(), C.data_ptr(), t.data_ptr(), 1, 1, n)
+        torch.cuda.synchronize()
+        K._check(fn)
+        assert np.array_equal(host(C), getattr(oracle, fn)(x, table))
+    oracle.set_threads(1)

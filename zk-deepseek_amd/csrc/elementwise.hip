@@ -6,6 +6,23 @@
 namespace zk {
 
 struct __attribute__((aligned(16))) i64x2 { int64_t x, y; };
+typedef int v4i_e __attribute__((ext_vector_type(4)));
+
+// Streaming 16-byte accesses (each byte is touched once): non-temporal, so they leave the caches alone.
+__device__ __forceinline__ i64x2 ld_stream(const i64x2 *p)
+{
+    v4i_e t = __builtin_nontemporal_load(reinterpret_cast<const v4i_e *>(p));
+    i64x2 r;
+    r.x = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
+    r.y = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
+    return r;
+}
+
+__device__ __forceinline__ void st_stream(i64x2 *p, i64x2 v)
+{
+    v4i_e t = { (int)(uint32_t)v.x, (int)(uint32_t)((uint64_t)v.x >> 32), (int)(uint32_t)v.y, (int)(uint32_t)((uint64_t)v.y >> 32) };
+    __builtin_nontemporal_store(t, reinterpret_cast<v4i_e *>(p));
+}
 
 // -------------------------------------------------------------------------------------------------
 // SiLU / sigmoid.  sigma(x) = 1 / (1 + e^-x) with e^-x = 2^y, y = -x*log2(e) split into an integer part
@@ -64,7 +81,7 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
             long i = base + (long)j * kActThreads;
-            if (i < nvec) v[j] = reinterpret_cast<const i64x2 *>(R)[i];
+            if (i < nvec) v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
         }
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
@@ -73,7 +90,7 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
                 i64x2 o;
                 o.x = act_one<Q, SIGMOID>(v[j].x, lut);
                 o.y = act_one<Q, SIGMOID>(v[j].y, lut);
-                reinterpret_cast<i64x2 *>(C)[i] = o;
+                st_stream(reinterpret_cast<i64x2 *>(C) + i, o);
             }
         }
         if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) C[n - 1] = act_one<Q, SIGMOID>(R[n - 1], lut);
@@ -87,6 +104,100 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
     }
 }
 
+// ---- large tensors: the reciprocal comes from a table ----------------------------------------------
+// sigma depends on x only through the shift k and the table index of the fraction, so for the 2Q+2 shifts in
+// [-(Q+1), Q] (every |x| below about 16.6 for Q23) the quotient 2^2Q / (2^Q + u) takes at most (2Q+2)*256
+// values.  A pre-kernel computes them from the caller's table with the same integer arithmetic as act_one;
+// the streaming kernel keeps them in LDS (48-52 KB) and does one 4-byte lookup per element instead of a
+// divide.  Elements outside that range, or a table whose quotients do not fit 32 bits, take act_one.
+template <int Q> struct QTab {
+    static constexpr int kLo = -(Q + 1), kHi = Q, kRows = kHi - kLo + 1, kEntries = kRows * 256;
+};
+
+template <int Q>
+__global__ __launch_bounds__(256) void act_qtab_kernel(const int64_t *__restrict__ lut, uint32_t *__restrict__ qtab,
+                                                       int *__restrict__ ok)
+{
+    constexpr int64_t ONE = (int64_t)1 << Q;
+    const int k = QTab<Q>::kLo + (int)blockIdx.x;
+    const int64_t t = lut[threadIdx.x];
+    int64_t u;
+    if (k < 0) u = t >> (-k);
+    else u = (int64_t)((uint64_t)t << k);
+    const int64_t den = (int64_t)((uint64_t)ONE + (uint64_t)u);
+    const int64_t q = tdiv64((int64_t)1 << (2 * Q), den);
+    qtab[blockIdx.x * 256 + threadIdx.x] = (uint32_t)q;
+    // one flag per shift row (no cross-workgroup traffic): 1 when every quotient of the row fits 32 bits
+    const int bad = __syncthreads_or(q < 0 || q > 0xFFFFFFFFll);
+    if (threadIdx.x == 0) ok[blockIdx.x] = bad ? 0 : 1;
+}
+
+constexpr int kTabThreads = 512;
+
+template <int Q, bool SIGMOID>
+__global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *__restrict__ R, int64_t *__restrict__ C,
+                                                                const int64_t *__restrict__ lut_g,
+                                                                const uint32_t *__restrict__ qtab_g,
+                                                                const int *__restrict__ ok_g, long n)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char act_smem[];
+    int64_t *lut = reinterpret_cast<int64_t *>(act_smem);
+    uint32_t *qtab = reinterpret_cast<uint32_t *>(act_smem + 2048);
+    constexpr int64_t LIM = (int64_t)64 << Q;
+    constexpr int64_t ONE = (int64_t)1 << Q;
+    if (threadIdx.x < 256) lut[threadIdx.x] = lut_g[threadIdx.x];
+    for (int i = threadIdx.x; i < QTab<Q>::kEntries / 4; i += kTabThreads)
+        reinterpret_cast<v4i_e *>(qtab)[i] = reinterpret_cast<const v4i_e *>(qtab_g)[i];
+    __shared__ int ok_s;
+    if (threadIdx.x == 0) {
+        int all = 1;
+        for (int i = 0; i < QTab<Q>::kRows; i++) all &= ok_g[i];
+        ok_s = all;
+    }
+    __syncthreads();
+    const bool ok = ok_s != 0;
+
+    auto one = [&](int64_t r) -> int64_t {
+        if (r >= LIM) return r;
+        if (r <= -LIM) return 0;
+        int64_t y;
+        if (Q == 23) y = ((-r) * ActConst<Q>::kLog2e) >> Q;
+        else y = -((r * ActConst<Q>::kLog2e) >> Q);
+        const int k = (int)(y >> Q);
+        if (!ok || k < QTab<Q>::kLo || k > QTab<Q>::kHi) return act_one<Q, SIGMOID>(r, lut);
+        const int idx = (int)((y & (ONE - 1)) >> (Q - 8));
+        const int64_t q = (int64_t)qtab[(k - QTab<Q>::kLo) * 256 + idx];
+        if (SIGMOID) return q;
+        return (r * q) >> Q;                 // |r| < 2^(Q+6), q <= 2^Q: exact in 64 bits
+    };
+
+    const long nvec = n >> 1;
+    const long stride = (long)gridDim.x * (kTabThreads * kActUnroll);
+    for (long base = (long)blockIdx.x * (kTabThreads * kActUnroll) + threadIdx.x; base < nvec; base += stride) {
+        i64x2 v[kActUnroll];
+#pragma unroll
+        for (int j = 0; j < kActUnroll; j++) {
+            long i = base + (long)j * kTabThreads;
+            if (i < nvec) v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
+        }
+#pragma unroll
+        for (int j = 0; j < kActUnroll; j++) {
+            long i = base + (long)j * kTabThreads;
+            if (i < nvec) {
+                i64x2 o;
+                o.x = one(v[j].x);
+                o.y = one(v[j].y);
+                st_stream(reinterpret_cast<i64x2 *>(C) + i, o);
+            }
+        }
+    }
+    if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) C[n - 1] = one(R[n - 1]);
+}
+
+static uint32_t *g_qtab = nullptr;      // (2Q+2)*256 quotients + the ok flag behind them, kept for the process lifetime
+constexpr size_t kQtabBytes = (size_t)QTab<25>::kEntries * 4;
+constexpr size_t kQtabFlagBytes = (size_t)QTab<25>::kRows * 4;
+
 template <int Q, bool SIGMOID>
 static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim)
 {
@@ -95,6 +206,32 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
     if (n == 0) return;
     if (!R || !C || !lut) { set_error(kBadArgument, "%s: null pointer", name); return; }
     bool vec = (((uintptr_t)R | (uintptr_t)C) & 15) == 0;
+    if (vec && n >= (1L << 20)) {
+        if (!g_qtab && hipMalloc(&g_qtab, kQtabBytes + kQtabFlagBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            g_qtab = nullptr;
+        }
+        if (g_qtab) {
+            int *ok = reinterpret_cast<int *>(reinterpret_cast<unsigned char *>(g_qtab) + kQtabBytes);
+            act_qtab_kernel<Q><<<dim3(QTab<Q>::kRows), dim3(256), 0, 0>>>(lut, g_qtab, ok);
+            const size_t lds = 2048 + (size_t)QTab<Q>::kEntries * 4;
+            static bool raised = false;
+            if (!raised) {
+                if (hipFuncSetAttribute((const void *)act_table_kernel<Q, SIGMOID>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds) != hipSuccess) {
+                    set_error(kLaunchFailure, "%s: cannot raise the LDS limit", name);
+                    return;
+                }
+                raised = true;
+            }
+            const long per_block = (long)kTabThreads * kActUnroll;
+            long blocks = ((n >> 1) + per_block - 1) / per_block;
+            if (blocks > 512) blocks = 512;            // persistent (2 per CU): each workgroup loads the table once
+            act_table_kernel<Q, SIGMOID><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, n);
+            check_launch(name);
+            return;
+        }
+    }
     long per_block = (long)kActThreads * kActUnroll;
     long items = vec ? ((n >> 1) > 0 ? (n >> 1) : 1) : n;
     long blocks = (items + per_block - 1) / per_block;

@@ -15,6 +15,24 @@ namespace zk {
 static bool g_softmax_clobber = false;
 
 struct __attribute__((aligned(16))) i64x2s { int64_t x, y; };
+typedef int v4i_s __attribute__((ext_vector_type(4)));
+
+// Streaming 16-byte accesses: every byte is touched exactly once, so the loads and stores are marked
+// non-temporal and do not displace anything from the caches.
+__device__ __forceinline__ i64x2s ld_stream(const i64x2s *p)
+{
+    v4i_s t = __builtin_nontemporal_load(reinterpret_cast<const v4i_s *>(p));
+    i64x2s r;
+    r.x = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
+    r.y = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
+    return r;
+}
+
+__device__ __forceinline__ void st_stream(i64x2s *p, i64x2s v)
+{
+    v4i_s t = { (int)(uint32_t)v.x, (int)(uint32_t)((uint64_t)v.x >> 32), (int)(uint32_t)v.y, (int)(uint32_t)((uint64_t)v.y >> 32) };
+    __builtin_nontemporal_store(t, reinterpret_cast<v4i_s *>(p));
+}
 
 template <int Q>
 __device__ __forceinline__ int64_t smx_weight(int64_t x, int64_t rmax, const int64_t *lut)
@@ -74,7 +92,7 @@ __global__ __launch_bounds__(kSmxThreads) void softmax_wave_kernel(int64_t *__re
         int idx = (j * 64 + lane) * 2;
         if (VEC) {
             if (idx < T) {
-                i64x2s p = *reinterpret_cast<const i64x2s *>(x + idx);
+                i64x2s p = ld_stream(reinterpret_cast<const i64x2s *>(x + idx));
                 v[2 * j] = p.x;
                 v[2 * j + 1] = p.y;
                 rmax = p.x > rmax ? p.x : rmax;
@@ -110,8 +128,8 @@ __global__ __launch_bounds__(kSmxThreads) void softmax_wave_kernel(int64_t *__re
                 w.y = v[2 * j + 1];
                 o.x = smx_norm<Q>(w.x, s, inv, fast);
                 o.y = smx_norm<Q>(w.y, s, inv, fast);
-                *reinterpret_cast<i64x2s *>(c + idx) = o;
-                if (clobber) *reinterpret_cast<i64x2s *>(x + idx) = w;
+                st_stream(reinterpret_cast<i64x2s *>(c + idx), o);
+                if (clobber) st_stream(reinterpret_cast<i64x2s *>(x + idx), w);
             }
         } else {
             if (idx < T) {
