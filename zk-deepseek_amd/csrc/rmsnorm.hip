@@ -186,8 +186,11 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
     if (i < N) C[row * N + i] = rms_apply_one(A[row * N + i], (int64_t)W[i], r, inv_r, fast_r);
 }
 
+typedef int v4i_r __attribute__((ext_vector_type(4)));
+
 // Statistic + normalisation, one workgroup per row, the row kept in registers (N <= 256 * EPT).
-template <typename WT, int EPT>
+// VEC: N is even and the rows are 16-byte aligned: elements are moved two at a time with streaming accesses.
+template <typename WT, int EPT, bool VEC>
 __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
                                                                 int64_t *__restrict__ rms, int64_t *__restrict__ C,
                                                                 int N, int64_t eps, int64_t dim)
@@ -198,10 +201,24 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     const int64_t *a = A + row * N;
     int64_t v[EPT];
     U192 acc = { 0, 0, 0 };
+    if (VEC) {
 #pragma unroll
-    for (int j = 0; j < EPT; j++) {
-        int i = j * kRmsThreads + threadIdx.x;
-        if (i < N) { v[j] = a[i]; u192_add_square(acc, v[j]); }
+        for (int j = 0; j < EPT / 2; j++) {
+            const int i = (j * kRmsThreads + threadIdx.x) * 2;
+            if (i < N) {
+                const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
+                v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
+                v[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
+                u192_add_square(acc, v[2 * j]);
+                u192_add_square(acc, v[2 * j + 1]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < EPT; j++) {
+            const int i = j * kRmsThreads + threadIdx.x;
+            if (i < N) { v[j] = a[i]; u192_add_square(acc, v[j]); }
+        }
     }
     U192 tot = block_sum_u192(acc, red);
     if (threadIdx.x == 0) {
@@ -213,10 +230,24 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     const int64_t r = rms_s;
     const bool fast_r = r > 0 && r < ((int64_t)1 << 62);
     const double inv_r = fast_r ? 1.0 / (double)r : 0.0;
+    if (VEC) {
 #pragma unroll
-    for (int j = 0; j < EPT; j++) {
-        int i = j * kRmsThreads + threadIdx.x;
-        if (i < N) C[row * N + i] = rms_apply_one(v[j], (int64_t)W[i], r, inv_r, fast_r);
+        for (int j = 0; j < EPT / 2; j++) {
+            const int i = (j * kRmsThreads + threadIdx.x) * 2;
+            if (i < N) {
+                const int64_t c0 = rms_apply_one(v[2 * j], (int64_t)W[i], r, inv_r, fast_r);
+                const int64_t c1 = rms_apply_one(v[2 * j + 1], (int64_t)W[i + 1], r, inv_r, fast_r);
+                const v4i_r t = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
+                                  (int)(uint32_t)((uint64_t)c1 >> 32) };
+                __builtin_nontemporal_store(t, reinterpret_cast<v4i_r *>(C + row * N + i));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < EPT; j++) {
+            const int i = j * kRmsThreads + threadIdx.x;
+            if (i < N) C[row * N + i] = rms_apply_one(v[j], (int64_t)W[i], r, inv_r, fast_r);
+        }
     }
 }
 
@@ -251,10 +282,17 @@ static void launch_fused(const char *name, const int64_t *A, const WT *W, int64_
 {
     if (!rms_args_ok(name, A, W, rms, C, M, N) || !stat_args_ok(name, eps, dim)) return;
     dim3 grid((unsigned)M), block(kRmsThreads);
-    if (N <= kRmsThreads * 2) rms_fused_kernel<WT, 2><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    else if (N <= kRmsThreads * 8) rms_fused_kernel<WT, 8><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    else if (N <= kRmsThreads * 32) rms_fused_kernel<WT, 32><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    else {
+    const bool vec = N % 2 == 0 && (((uintptr_t)A | (uintptr_t)C) & 15) == 0;
+    if (N <= kRmsThreads * 2) {
+        if (vec) rms_fused_kernel<WT, 2, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+        else rms_fused_kernel<WT, 2, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+    } else if (N <= kRmsThreads * 8) {
+        if (vec) rms_fused_kernel<WT, 8, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+        else rms_fused_kernel<WT, 8, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+    } else if (N <= kRmsThreads * 32) {
+        if (vec) rms_fused_kernel<WT, 32, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+        else rms_fused_kernel<WT, 32, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
+    } else {
         rms_stat_kernel<<<grid, block, 0, 0>>>(A, rms, N, eps, dim);
         if (check_launch(name)) launch_apply<WT>(name, A, W, rms, C, M, N);
         return;
