@@ -36,6 +36,9 @@
 #ifndef ZK_PREFETCH
 #define ZK_PREFETCH 0
 #endif
+#ifndef ZK_NARROW_LAYOUT
+#define ZK_NARROW_LAYOUT 0
+#endif
 #ifndef ZK_KK
 #define ZK_KK(DD) 1
 #endif
@@ -57,7 +60,10 @@ struct MfmaParams {
     int verify_b_all_batches;       // B differs per batch: every batch's first tile row tracks its range
     const unsigned char *a_planes;  // pre-split digits of A (planes variants only)
     int a_msub, a_ksteps;           // 32-row groups and 32-k steps the planes were written for
-    int dbg;
+    // split-K tail: workgroup ids below main_tiles are whole tiles; the rest are `split` workgroups per tile that
+    // each cover a slice of K and leave raw 128-bit partial sums in `partials`
+    int main_tiles, split;
+    unsigned long long *partials;
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -285,22 +291,31 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
     }
 }
 
-// Folds the per-workgroup ranges of the pre-pass into range[0..1].
+// Folds the per-workgroup ranges of the pre-pass into range[0..1] and resets the B slots range[2..3].
 __global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long long *mm, long count, unsigned long long *range)
 {
-    __shared__ unsigned long long lo_s[256], hi_s[256];
+    __shared__ unsigned long long lo_s[4], hi_s[4];
     unsigned long long lo = ~0ull, hi = 0ull;
     for (long i = threadIdx.x; i < count; i += 256) {
-        lo = mm[2 * i] < lo ? mm[2 * i] : lo;
-        hi = mm[2 * i + 1] > hi ? mm[2 * i + 1] : hi;
+        const unsigned long long a = mm[2 * i], b = mm[2 * i + 1];
+        lo = a < lo ? a : lo;
+        hi = b > hi ? b : hi;
     }
-    lo_s[threadIdx.x] = lo;
-    hi_s[threadIdx.x] = hi;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long ol = (unsigned long long)__shfl_xor((long long)lo, off, kWave);
+        const unsigned long long oh = (unsigned long long)__shfl_xor((long long)hi, off, kWave);
+        lo = ol < lo ? ol : lo;
+        hi = oh > hi ? oh : hi;
+    }
+    if ((threadIdx.x & 63) == 0) { lo_s[threadIdx.x >> 6] = lo; hi_s[threadIdx.x >> 6] = hi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < 256; i++) { lo = lo_s[i] < lo ? lo_s[i] : lo; hi = hi_s[i] > hi ? hi_s[i] : hi; }
+        for (int i = 1; i < 4; i++) { lo = lo_s[i] < lo ? lo_s[i] : lo; hi = hi_s[i] > hi ? hi_s[i] : hi; }
         range[0] = lo;
         range[1] = hi;
+        range[2] = ~0ull;
+        range[3] = 0ull;
     }
 }
 
@@ -331,9 +346,16 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     // ids are regrouped to give each XCD a contiguous run of tiles; within a run the tile-row index moves
     // fastest, so the workgroups that share a B tile sit on the same L2.
     const int per_batch = p.tiles_m * p.tiles_n;
-    const int total = per_batch * gridDim.y;
-    int lin = blockIdx.y * per_batch + blockIdx.x;
-    if ((total & 7) == 0) lin = (lin & 7) * (total >> 3) + (lin >> 3);
+    int lin = blockIdx.x, sidx = 0, nsplit = 1;
+    if (lin < p.main_tiles) {
+        if ((p.main_tiles & 7) == 0) lin = (lin & 7) * (p.main_tiles >> 3) + (lin >> 3);
+    } else {
+        const int t = lin - p.main_tiles;
+        lin = p.main_tiles + t / p.split;
+        sidx = t % p.split;
+        nsplit = p.split;
+    }
+    const int tail_tile = lin - p.main_tiles;      // index among the split tiles (when nsplit > 1)
     const int g = lin / per_batch;
     const int rem = lin - g * per_batch;
     const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
@@ -555,6 +577,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
     const int ksteps = (p.K + BK - 1) / BK;
     const int full_steps = (a_vec || APL) && (b_vec || BKM) ? p.K / BK : 0;     // steps that can use unguarded loads
+    // this workgroup's slice of the k-steps (everything unless it is one of the split workgroups of a tail tile)
+    const int ks_begin = (int)((long)sidx * ksteps / nsplit), ks_end = (int)((long)(sidx + 1) * ksteps / nsplit);
 
     // Range tracking of the staged elements of data step d, done while the registers still hold them.
     auto track = [&](int d) {
@@ -578,7 +602,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     //      elements staged for step ks+1 and their LDS writes into the other stage;
     //   C  the loads of step ks+2 into the now free staging registers, then the barrier.
     auto step_body = [&](int ks, auto fast_tag) {
-        const int cur = ks & 1;
+        const int cur = (ks - ks_begin) & 1;
 #pragma unroll
         for (int kk = 0; kk < KK - 1; kk++) {
             v4i fa[WM][NA], fb[WN][NB];
@@ -599,21 +623,24 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         }
         __builtin_amdgcn_sched_barrier(0);
         track(ks + 1);
-        if (ks + 2 < ksteps) fetch(ks + 2, fast_tag);
+        if (ks + 2 < ks_end) fetch(ks + 2, fast_tag);
         if (ZK_PREFETCH > 0 && decltype(fast_tag)::value && ks + 2 + ZK_PREFETCH < full_steps) prefetch(ks + 2 + ZK_PREFETCH);
         __syncthreads();
     };
 
-    // prologue: stage 0 holds step 0, the staging registers hold step 1
-    if (full_steps > 0) fetch(0, std::true_type()); else fetch(0, std::false_type());
-    track(0);
+    // prologue: stage 0 holds the first step, the staging registers hold the second
+    if (ks_begin < full_steps) fetch(ks_begin, std::true_type()); else fetch(ks_begin, std::false_type());
+    track(ks_begin);
     stash(0);
-    if (ksteps > 1) { if (full_steps > 1) fetch(1, std::true_type()); else fetch(1, std::false_type()); }
+    if (ks_begin + 1 < ks_end) {
+        if (ks_begin + 1 < full_steps) fetch(ks_begin + 1, std::true_type()); else fetch(ks_begin + 1, std::false_type());
+    }
     __syncthreads();
-    int ks = 0;
-    for (; ks + 2 < full_steps; ks++) step_body(ks, std::true_type());
-    for (; ks + 1 < ksteps; ks++) step_body(ks, std::false_type());
-    compute_all((ksteps - 1) & 1);
+    int ks = ks_begin;
+    const int fast_end = full_steps < ks_end ? full_steps : ks_end;
+    for (; ks + 2 < fast_end; ks++) step_body(ks, std::true_type());
+    for (; ks + 1 < ks_end; ks++) step_body(ks, std::false_type());
+    compute_all((ks_end - 1 - ks_begin) & 1);
 
     if (verify_a) mm_publish(ra, p.range);
     if (verify_b) mm_publish(rb, p.range + 2);
@@ -630,7 +657,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                uint64_t lo = (uint64_t)p.init, hi = (uint64_t)(p.init >> 63);
+                // whole tiles start from the rounding term; split workgroups leave it to the finishing kernel
+                uint64_t lo = nsplit > 1 ? 0 : (uint64_t)p.init, hi = nsplit > 1 ? 0 : (uint64_t)(p.init >> 63);
 #pragma unroll
                 for (int d = 0; d < D; d++) {
                     const int64_t v = (int64_t)acc[a][b][d][r];
@@ -643,7 +671,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                     hi += chi + (s < lo ? 1 : 0);
                     lo = s;
                 }
-                if (m < p.M && n < p.N) {
+                if (nsplit > 1) {
+                    // raw partial sum (without init): 16 bytes per output, lane-contiguous, finished by
+                    // gemm_split_finish_kernel
+                    const long e = ((((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r) * 64 + lane;
+                    p.partials[2 * e] = lo;
+                    p.partials[2 * e + 1] = hi;
+                } else if (m < p.M && n < p.N) {
                     const long o = (long)g * p.sC + (long)m * p.ldc + n;
                     uint64_t q;
                     if (p.shift == 0) q = lo;
@@ -656,6 +690,46 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     }
 }
 
+// Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
+// Thread layout and element order are those of the GEMM kernel's epilogue.
+template <int WVM, int WVN, int WM, int WN>
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaParams p)
+{
+    constexpr int T = 64 * WVM * WVN, BM = 32 * WM * WVM, BN = 32 * WN * WVN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WVN, wn = wave % WVN;
+    const int per_batch = p.tiles_m * p.tiles_n;
+    const int tail_tile = blockIdx.x >> 2, rq = blockIdx.x & 3, lin = p.main_tiles + tail_tile;
+    const int g = lin / per_batch, rem = lin - g * per_batch;
+    const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+#pragma unroll
+    for (int a = 0; a < WM; a++)
+#pragma unroll
+        for (int b = 0; b < WN; b++) {
+            const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int r = rq * 4 + r4;
+                const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                uint64_t lo = (uint64_t)p.init, hi = (uint64_t)(p.init >> 63);
+                for (int sidx = 0; sidx < p.split; sidx++) {
+                    const long e = ((((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r) * 64 + lane;
+                    const uint64_t plo = p.partials[2 * e], phi = p.partials[2 * e + 1];
+                    const uint64_t s = lo + plo;
+                    hi += phi + (s < lo ? 1 : 0);
+                    lo = s;
+                }
+                if (m < p.M && n < p.N) {
+                    const long o = (long)g * p.sC + (long)m * p.ldc + n;
+                    p.C[o] = (int64_t)(p.shift == 0 ? lo : ((lo >> p.shift) | (hi << (64 - p.shift))));
+                    if (p.R) p.R[o] = (int64_t)(lo & rmask);
+                }
+            }
+        }
+}
+
 // ---- host side ---------------------------------------------------------------------------------------
 typedef void (*MfmaKernel)(MfmaParams);
 typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
@@ -666,6 +740,7 @@ struct Instance {
     int na, nb, bm, bn, threads, kk;
     MfmaKernel fn[kVariants];
     PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
+    MfmaKernel finish;           // adds up the partial sums of split tail tiles
 };
 
 
@@ -675,9 +750,16 @@ static Instance make_instance()
     constexpr int DD = NA + NB - 1;
     // narrow: 8 waves as 2x4, 64x32 per wave (128x128); mid: 8 waves as 4x2, 32x32 per wave (128x64);
     // wide: 4 waves as 2x2, 32x32 per wave (64x64, one wave per SIMD because of the accumulator count)
+#if ZK_NARROW_LAYOUT == 1
+    // narrow: 12 waves as 4x3, 32x32 per wave (128x96), three waves per SIMD
+    constexpr int WVM = DD <= 5 ? 4 : (DD <= 10 ? 4 : 2);
+    constexpr int WVN = DD <= 5 ? 3 : 2;
+    constexpr int WM = 1, WN = 1;
+#else
     constexpr int WVM = DD <= 5 ? 2 : (DD <= 10 ? 4 : 2);
     constexpr int WVN = DD <= 5 ? 4 : 2;
     constexpr int WM = DD <= 5 ? 2 : 1, WN = 1;
+#endif
     constexpr int KK = ZK_KK(DD);
     Instance s;
     s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
@@ -690,6 +772,7 @@ static Instance make_instance()
         s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true>;
         s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false>;
     }
+    s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
     s.planes[0] = a_planes_kernel<NA, 2, KK>;
     s.planes[1] = a_planes_kernel<NA, 4, KK>;
     return s;
@@ -734,6 +817,9 @@ struct RangeCache {
     size_t planes_bytes = 0;
     unsigned long long *mm = nullptr;        // per-workgroup ranges of the plane pre-pass
     size_t mm_count = 0;
+    unsigned long long *partials = nullptr;  // 128-bit partial sums of split tail tiles
+    size_t partials_bytes = 0;
+    int cus = 0;                             // compute units of the device
     int lookup(const void *ptr, long rows, long K, int esz)
     {
         auto it = limbs.find(std::make_tuple(ptr, rows, K, esz));
@@ -777,7 +863,12 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     p.range = g_cache.dev;
     p.verify_b_all_batches = d.sB != 0;
     p.a_planes = nullptr; p.a_msub = 0; p.a_ksteps = 0;
-    p.dbg = 0;
+    p.main_tiles = 0; p.split = 1; p.partials = nullptr;
+    if (!g_cache.cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        g_cache.cus = n;
+    }
 
     const long rows_a = (long)d.G * d.M;
     int na = g_cache.lookup(d.A, rows_a, d.K, 8);
@@ -810,7 +901,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
         if (!fn) return false;
-        range_reset_kernel<<<1, 64, 0, 0>>>(p.range);
+        if (!use_planes) range_reset_kernel<<<1, 64, 0, 0>>>(p.range);       // with planes the fold kernel does it
         if (use_planes) {
             const int msub = p.tiles_m * (BM / 32);
             const size_t need = (size_t)d.G * msub * ksteps * inst->na * 1024;
@@ -856,8 +947,45 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             }
             lds_raised.insert((const void *)fn);
         }
-        fn<<<dim3((unsigned)per_batch, (unsigned)d.G), dim3((unsigned)inst->threads), lds, 0>>>(p);
+        // Tail split: with `total` tiles on `cus` compute units the last partial round would leave most of the
+        // device idle.  Its tiles are cut into `split` slices of K each, run as extra workgroups in the same
+        // launch, and a small kernel adds the 128-bit partial sums.
+        const long total = per_batch * d.G;
+        if (total > 0x7FFFFFFFL / 8) return false;
+        const int tail = (int)(total % g_cache.cus);
+        p.main_tiles = (int)total;
+        p.split = 1;
+        if (total > g_cache.cus && tail > 0 && tail <= g_cache.cus / 2 && getenv("ZK_NO_TAIL_SPLIT") == nullptr) {
+            int split = g_cache.cus / tail;
+            if (split > 8) split = 8;
+            const int steps = (d.K + 32 * inst->kk - 1) / (32 * inst->kk);
+            if (split > steps / 8) split = steps / 8;
+            if (split >= 2) {
+                const size_t need = (size_t)tail * split * BM * BN * 16;
+                if (need > g_cache.partials_bytes) {
+                    if (g_cache.partials && hipFree(g_cache.partials) != hipSuccess) {
+                        set_error(kLaunchFailure, "gemm: cannot release the partial-sum buffer");
+                        return false;
+                    }
+                    g_cache.partials = nullptr;
+                    g_cache.partials_bytes = 0;
+                    if (hipMalloc(&g_cache.partials, need) == hipSuccess) g_cache.partials_bytes = need;
+                    else (void)hipGetLastError();
+                }
+                if (g_cache.partials) {
+                    p.main_tiles = (int)(total - tail);
+                    p.split = split;
+                    p.partials = g_cache.partials;
+                }
+            }
+        }
+        const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
+        fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
+        if (p.split > 1) {
+            inst->finish<<<dim3((unsigned)(total - p.main_tiles) * 4), dim3((unsigned)inst->threads), 0, 0>>>(p);
+            if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
+        }
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
