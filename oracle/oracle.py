@@ -48,6 +48,8 @@ def _load():
         getattr(lib, name).argtypes = [vp, vp, vp, vp, ci, ci, ci, ci]
     for name in ("ora_act_q23", "ora_act_q25"):
         getattr(lib, name).argtypes = [vp, vp, vp, cl, ci]
+    lib.ora_bf16_to_int32.argtypes = [vp, vp, cl, ci, ci]
+    lib.ora_float32_to_int64.argtypes = [vp, vp, cl, ci]
     lib.ora_set_threads.argtypes = [ci]
     lib.ora_max_threads.restype = ci
     return lib
@@ -228,3 +230,25 @@ def silu_q25(R, lut=None):
 
 def sigmoid_q25(R, lut=None):
     return _act(_lib.ora_act_q25, R, silu_init_q25() if lut is None else lut, 1)
+
+
+def bf16_to_int32_2d(bits, rescale):
+    """bits: uint16 bf16 patterns [rows, cols] -> int32 fixed point (inference/int64_gemm.cu:92-132)"""
+    bits = _c(bits, np.uint16)
+    out = np.empty(bits.shape, np.int32)
+    _lib.ora_bf16_to_int32(_p(bits), _p(out), bits.size, rescale, 0)
+    return out
+
+
+def wkv_b_bf16_to_int32(bits):
+    bits = _c(bits, np.uint16)
+    out = np.empty(bits.shape, np.int32)
+    _lib.ora_bf16_to_int32(_p(bits), _p(out), bits.size, 25, 1)
+    return out
+
+
+def float32_to_int64_2d(bits, rescale):
+    bits = _c(bits, np.uint32)
+    out = np.empty(bits.shape, np.int64)
+    _lib.ora_float32_to_int64(_p(bits), _p(out), bits.size, rescale)
+    return out

@@ -438,3 +438,45 @@ void ora_act_q25(const int64_t *Rin, int64_t *C, const int64_t *lut, long n, int
         C[i] = mode ? q : (int64_t)((uint64_t)r * (uint64_t)q) >> 25;
     }
 }
+
+/* ---- float bit patterns -> fixed point (exported by the reference, bound by none of its Python) ---------
+ * inference/int64_gemm.cu:92-132 (bf16 -> int32), :134-179 (wkv_b variant: 2^25 scale, saturates |x| >= 0.5),
+ * :181-221 (fp32 -> int64).  value = (1.mantissa) * 2^(exp + rescale), truncated toward zero, sign applied last.
+ * The reference forms `1 << ex2` in 32-bit int: shifts of 32 or more are hardware-defined there; here a left
+ * shift of 32 or more multiplies by 0 and a right shift of 31 or more divides to 0 (parity unpinned). */
+static uint32_t scale_mantissa_u32(uint32_t r2, int ex2)
+{
+    if (ex2 >= 0) return ex2 >= 32 ? 0u : r2 * (1u << ex2);
+    return -ex2 >= 31 ? 0u : r2 / (1u << -ex2);
+}
+
+void ora_bf16_to_int32(const uint16_t *in, int32_t *out, long n, int rescale, int wkv_b)
+{
+    for (long i = 0; i < n; i++) {
+        int v0 = in[i];
+        int ex0 = ((v0 >> 7) & 0xFF) - 127;
+        int r0 = v0 & 0x7F;
+        if (ex0 == -127 && r0 == 0) { out[i] = 0; continue; }                 /* :104-107 */
+        if (wkv_b && ex0 >= -1) { out[i] = 0x7FFFFFFF; continue; }            /* :151-154 */
+        uint32_t v = scale_mantissa_u32((uint32_t)(r0 + 128), ex0 + rescale); /* :109-116 */
+        if (v0 & 0x8000) v = 0u - v;                                          /* :118-120 */
+        out[i] = (int32_t)v;
+    }
+}
+
+void ora_float32_to_int64(const uint32_t *in, int64_t *out, long n, int rescale)
+{
+    for (long i = 0; i < n; i++) {
+        uint32_t v0 = in[i];
+        int ex0 = (int)((v0 >> 23) & 0xFF) - 127;
+        int r0 = (int)(v0 & 0x7FFFFF);
+        if (ex0 == -127 && r0 == 0) { out[i] = 0; continue; }
+        int ex2 = ex0 + rescale;
+        int64_t r2 = (int64_t)r0 + 8388608;
+        int64_t v;
+        if (ex2 >= 0) v = ex2 >= 32 ? 0 : (int64_t)((uint64_t)r2 * (uint64_t)(int64_t)(int32_t)(1u << ex2));   /* :202 */
+        else v = -ex2 >= 31 ? 0 : r2 / (int64_t)(1u << -ex2);                                                   /* :204 */
+        if (v0 & 0x80000000u) v = (int64_t)(0 - (uint64_t)v);
+        out[i] = v;
+    }
+}

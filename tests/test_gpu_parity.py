@@ -436,3 +436,23 @@ def test_activation_table_path(K, oracle, fn, Q):
         K._check(fn)
         assert np.array_equal(host(C), getattr(oracle, fn)(x, table))
     oracle.set_threads(1)
+
+
+def test_converters(K, oracle):
+    """the three float -> fixed converters the reference exports (inference/int64_gemm.cu:92-221)"""
+    rng = np.random.default_rng(31)
+    bits32 = rng.integers(0, 1 << 32, size=(37, 129), dtype=np.uint64).astype(np.uint32)
+    bits16 = rng.integers(0, 1 << 16, size=(37, 129), dtype=np.uint64).astype(np.uint16)
+    for rescale in (0, 12, 25, 40):
+        o64 = torch.empty((37, 129), dtype=torch.int64, device="cuda")
+        src = torch.from_numpy(bits32.view(np.int32)).cuda()
+        K.lib.float32_to_int64_2d(src.data_ptr(), o64.data_ptr(), 37, 129, rescale)
+        assert np.array_equal(host(o64), oracle.float32_to_int64_2d(bits32, rescale))
+        o32 = torch.empty((37, 129), dtype=torch.int32, device="cuda")
+        src16 = torch.from_numpy(bits16.view(np.int16)).cuda()
+        K.lib.bf16_to_int32_2d(src16.data_ptr(), o32.data_ptr(), 37, 129, rescale)
+        assert np.array_equal(host(o32), oracle.bf16_to_int32_2d(bits16, rescale))
+    o32 = torch.empty((37, 129), dtype=torch.int32, device="cuda")
+    K.lib.wkv_b_bf16_to_int32(src16.data_ptr(), o32.data_ptr(), 37, 129)
+    assert np.array_equal(host(o32), oracle.wkv_b_bf16_to_int32(bits16))
+    K._check("converters")

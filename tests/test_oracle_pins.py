@@ -290,3 +290,46 @@ def test_sigmoid_q23_hand_steps(oracle):
     assert oracle.sigmoid_q23(x)[0] == (1 << 46) // ((1 << 23) + (int(lut[255]) >> 1))    # y = -5 -> k=-1, f=2^23-5
     lut25 = oracle.silu_init_q25()
     assert oracle.sigmoid_q25(x)[0] == (1 << 50) // ((1 << 25) + (int(lut25[255]) >> 1))   # y = -(4) -> k=-1
+
+
+# -------------------------------------------------------------------- float -> fixed converters ---
+def test_converters_truncate_the_scaled_float(oracle):
+    """the converters scale the INTEGER mantissa (1.m * 2^23 for fp32, 1.m * 2^7 for bf16) by 2^(exp + rescale), so
+    the value is trunc(|x| * 2^(rescale + 23)) resp. trunc(|x| * 2^(rescale + 7)) with the sign applied afterwards:
+    checked against exact rational arithmetic wherever the 32-bit shift of the reference is defined"""
+    from fractions import Fraction
+    rng = np.random.default_rng(77)
+    f = (rng.standard_normal(4000) * np.exp(rng.uniform(-12, 6, 4000))).astype(np.float32)
+    f[:6] = [0.0, -0.0, 1.0, -1.0, 0.5, -0.4999]
+    bits32 = f.view(np.uint32)
+    checked = 0
+    for rescale in (-20, -3, 0, 8):
+        out = oracle.float32_to_int64_2d(bits32.reshape(40, 100), rescale).ravel()
+        for x, o in zip(f.tolist(), out.tolist()):
+            if x == 0:
+                assert o == 0
+                continue
+            ex2 = int(np.frexp(np.float32(x))[1]) - 1 + rescale
+            if -31 < ex2 < 31 and abs(x) >= 2.0 ** -126:
+                want = int(abs(Fraction(x)) * Fraction(2) ** (rescale + 23))
+                assert o == (want if x > 0 else -want), (x, rescale)
+                checked += 1
+    assert checked > 8000
+    bf = (bits32 >> 16).astype(np.uint16)                          # truncating fp32 -> bf16 gives valid bf16 patterns
+    fb = (bf.astype(np.uint32) << 16).view(np.float32)
+    out = oracle.bf16_to_int32_2d(bf.reshape(40, 100), 12).ravel()
+    for x, o in zip(fb.tolist(), out.tolist()):
+        if x == 0:
+            assert o == 0
+            continue
+        ex2 = int(np.frexp(np.float32(x))[1]) - 1 + 12
+        if -31 < ex2 < 24 and abs(x) >= 2.0 ** -126:
+            want = int(abs(Fraction(x)) * Fraction(2) ** (12 + 7))
+            assert o == (want if x > 0 else -want), x
+    sat = oracle.wkv_b_bf16_to_int32(bf.reshape(40, 100)).ravel()
+    plain = oracle.bf16_to_int32_2d(bf.reshape(40, 100), 25).ravel()
+    for x, o, pl in zip(fb.tolist(), sat.tolist(), plain.tolist()):
+        if abs(x) >= 0.5:
+            assert o == 0x7FFFFFFF                                 # saturates regardless of sign (:151-154)
+        else:
+            assert o == pl                                         # otherwise the rescale-25 conversion

@@ -64,6 +64,7 @@ struct MfmaParams {
     // each cover a slice of K and leave raw 128-bit partial sums in `partials`
     int main_tiles, split;
     unsigned long long *partials;
+    int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -149,6 +150,16 @@ __device__ __forceinline__ MinMax mm_wave(MinMax r)
         r.hi = oh > r.hi ? oh : r.hi;
     }
     return r;
+}
+
+// single-lane publish of an already reduced range
+__device__ __forceinline__ void mm_publish_lane(MinMax r, unsigned long long *slot)
+{
+    const unsigned long long lo = (unsigned long long)r.lo ^ kSignFlip, hi = (unsigned long long)r.hi ^ kSignFlip;
+    if (r.lo <= r.hi) {
+        if (lo < __atomic_load_n(slot, __ATOMIC_RELAXED)) atomicMin(slot, lo);
+        if (hi > __atomic_load_n(slot + 1, __ATOMIC_RELAXED)) atomicMax(slot + 1, hi);
+    }
 }
 
 __device__ __forceinline__ void mm_publish(MinMax r, unsigned long long *slot)
@@ -642,8 +653,23 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     for (; ks + 1 < ks_end; ks++) step_body(ks, std::false_type());
     compute_all((ks_end - 1 - ks_begin) & 1);
 
-    if (verify_a) mm_publish(ra, p.range);
-    if (verify_b) mm_publish(rb, p.range + 2);
+    // one publishing lane per workgroup: the waves' ranges meet in LDS (the stages are free by now)
+    if (verify_a || verify_b) {
+        __syncthreads();
+        MinMax *red = reinterpret_cast<MinMax *>(smem);
+        ra = mm_wave(ra);
+        rb = mm_wave(rb);
+        if (lane == 0) { red[2 * wave] = ra; red[2 * wave + 1] = rb; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < T / 64; w++) {
+                mm_update(ra, red[2 * w].lo); mm_update(ra, red[2 * w].hi);
+                mm_update(rb, red[2 * w + 1].lo); mm_update(rb, red[2 * w + 1].hi);
+            }
+            if (verify_a) mm_publish_lane(ra, p.range);
+            if (verify_b) mm_publish_lane(rb, p.range + 2);
+        }
+    }
     if (pf_acc == 0x7f3a91c5 && p.shift == 99) p.C[0] = pf_acc;      // never true: keeps the warm-up loads alive
 
     // epilogue: diagonals -> 128-bit sum -> shift.  Accumulator register r of lane l holds
@@ -699,7 +725,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WVN, wn = wave % WVN;
     const int per_batch = p.tiles_m * p.tiles_n;
-    const int tail_tile = blockIdx.x >> 2, rq = blockIdx.x & 3, lin = p.main_tiles + tail_tile;
+    const int tail_tile = blockIdx.x / p.finish_rq, rq = blockIdx.x % p.finish_rq, lin = p.main_tiles + tail_tile;
+    const int r_per = 16 / p.finish_rq;
     const int g = lin / per_batch, rem = lin - g * per_batch;
     const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
@@ -709,9 +736,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
 #pragma unroll
         for (int b = 0; b < WN; b++) {
             const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                const int r = rq * 4 + r4;
+            for (int r4 = 0; r4 < r_per; r4++) {
+                const int r = rq * r_per + r4;
                 const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 uint64_t lo = (uint64_t)p.init, hi = (uint64_t)(p.init >> 63);
                 for (int sidx = 0; sidx < p.split; sidx++) {
@@ -738,31 +764,35 @@ enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32
 
 struct Instance {
     int na, nb, bm, bn, threads, kk;
+    bool skinny;                 // 32-row tiles for M <= 32
     MfmaKernel fn[kVariants];
     PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
     MfmaKernel finish;           // adds up the partial sums of split tail tiles
 };
 
 
-template <int NA, int NB>
+template <int NA, int NB, bool SKINNY = false>
 static Instance make_instance()
 {
     constexpr int DD = NA + NB - 1;
+    static_assert(!SKINNY || DD <= 10, "skinny tiles keep two waves per SIMD");
     // narrow: 8 waves as 2x4, 64x32 per wave (128x128); mid: 8 waves as 4x2, 32x32 per wave (128x64);
     // wide: 4 waves as 2x2, 32x32 per wave (64x64, one wave per SIMD because of the accumulator count)
-#if ZK_NARROW_LAYOUT == 1
+#if 0
     // narrow: 12 waves as 4x3, 32x32 per wave (128x96), three waves per SIMD
     constexpr int WVM = DD <= 5 ? 4 : (DD <= 10 ? 4 : 2);
     constexpr int WVN = DD <= 5 ? 3 : 2;
     constexpr int WM = 1, WN = 1;
 #else
-    constexpr int WVM = DD <= 5 ? 2 : (DD <= 10 ? 4 : 2);
-    constexpr int WVN = DD <= 5 ? 4 : 2;
-    constexpr int WM = DD <= 5 ? 2 : 1, WN = 1;
+    // skinny (M <= 32): 8 waves as 1x8, 32x32 per wave (32x256)
+    constexpr int WVM = SKINNY ? 1 : (DD <= 5 ? 2 : (DD <= 10 ? 4 : 2));
+    constexpr int WVN = SKINNY ? 8 : (DD <= 5 ? 4 : 2);
+    constexpr int WM = SKINNY ? 1 : (DD <= 5 ? 2 : 1), WN = 1;
 #endif
     constexpr int KK = ZK_KK(DD);
     Instance s;
     s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
+    s.skinny = SKINNY;
     for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
     s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false>;
     s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true>;
@@ -788,20 +818,21 @@ static const Instance *instances(int *count)
         make_instance<3, 3>(), make_instance<4, 3>(), make_instance<4, 4>(), make_instance<5, 4>(),
         make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(),
         make_instance<9, 5>(), make_instance<5, 9>(), make_instance<9, 9>(),
+        make_instance<3, 3, true>(), make_instance<5, 5, true>(),
 #endif
     };
     *count = (int)(sizeof(table) / sizeof(table[0]));
     return table;
 }
 
-static const Instance *pick_instance(int na, int nb, bool b32)
+static const Instance *pick_instance(int na, int nb, bool b32, bool skinny)
 {
     int count;
     const Instance *t = instances(&count);
     const Instance *best = nullptr;
     long best_cost = 0;
     for (int i = 0; i < count; i++) {
-        if (t[i].na < na || t[i].nb < nb) continue;
+        if (t[i].na < na || t[i].nb < nb || t[i].skinny != skinny) continue;
         if (b32 && !t[i].fn[kB32Fly]) continue;
         long cost = (long)t[i].na * t[i].nb;
         if (!best || cost < best_cost) { best = &t[i]; best_cost = cost; }
@@ -863,7 +894,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     p.range = g_cache.dev;
     p.verify_b_all_batches = d.sB != 0;
     p.a_planes = nullptr; p.a_msub = 0; p.a_ksteps = 0;
-    p.main_tiles = 0; p.split = 1; p.partials = nullptr;
+    p.main_tiles = 0; p.split = 1; p.partials = nullptr; p.finish_rq = 4;
     if (!g_cache.cus) {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
@@ -884,7 +915,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     }
 
     for (int attempt = 0; attempt < 3; attempt++) {
-        const Instance *inst = pick_instance(na, nb, d.b32 != 0);
+        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true) : nullptr;
+        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false);
         if (!inst) return false;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
@@ -952,38 +984,48 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         // launch, and a small kernel adds the 128-bit partial sums.
         const long total = per_batch * d.G;
         if (total > 0x7FFFFFFFL / 8) return false;
-        const int tail = (int)(total % g_cache.cus);
+        // A launch smaller than the device is split the same way over all of its tiles.
+        const int steps = (d.K + 32 * inst->kk - 1) / (32 * inst->kk);
+        int tail = (int)(total % g_cache.cus), split = 1;
         p.main_tiles = (int)total;
         p.split = 1;
-        if (total > g_cache.cus && tail > 0 && tail <= g_cache.cus / 2 && getenv("ZK_NO_TAIL_SPLIT") == nullptr) {
-            int split = g_cache.cus / tail;
-            if (split > 8) split = 8;
-            const int steps = (d.K + 32 * inst->kk - 1) / (32 * inst->kk);
-            if (split > steps / 8) split = steps / 8;
-            if (split >= 2) {
-                const size_t need = (size_t)tail * split * BM * BN * 16;
-                if (need > g_cache.partials_bytes) {
-                    if (g_cache.partials && hipFree(g_cache.partials) != hipSuccess) {
-                        set_error(kLaunchFailure, "gemm: cannot release the partial-sum buffer");
-                        return false;
-                    }
-                    g_cache.partials = nullptr;
-                    g_cache.partials_bytes = 0;
-                    if (hipMalloc(&g_cache.partials, need) == hipSuccess) g_cache.partials_bytes = need;
-                    else (void)hipGetLastError();
+        p.finish_rq = 4;
+        if (getenv("ZK_NO_TAIL_SPLIT") == nullptr) {
+            if (total < g_cache.cus) {
+                tail = (int)total;
+                split = g_cache.cus / tail;
+                if (split > 64) split = 64;
+                if (split > steps / 4) split = steps / 4;
+                p.finish_rq = 16;
+            } else if (tail > 0 && tail <= g_cache.cus / 2) {
+                split = g_cache.cus / tail;
+                if (split > 8) split = 8;
+                if (split > steps / 8) split = steps / 8;
+            }
+        }
+        if (split >= 2) {
+            const size_t need = (size_t)tail * split * BM * BN * 16;
+            if (need > g_cache.partials_bytes) {
+                if (g_cache.partials && hipFree(g_cache.partials) != hipSuccess) {
+                    set_error(kLaunchFailure, "gemm: cannot release the partial-sum buffer");
+                    return false;
                 }
-                if (g_cache.partials) {
-                    p.main_tiles = (int)(total - tail);
-                    p.split = split;
-                    p.partials = g_cache.partials;
-                }
+                g_cache.partials = nullptr;
+                g_cache.partials_bytes = 0;
+                if (hipMalloc(&g_cache.partials, need) == hipSuccess) g_cache.partials_bytes = need;
+                else (void)hipGetLastError();
+            }
+            if (g_cache.partials) {
+                p.main_tiles = (int)(total - tail);
+                p.split = split;
+                p.partials = g_cache.partials;
             }
         }
         const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
         if (p.split > 1) {
-            inst->finish<<<dim3((unsigned)(total - p.main_tiles) * 4), dim3((unsigned)inst->threads), 0, 0>>>(p);
+            inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq)), dim3((unsigned)inst->threads), 0, 0>>>(p);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
         }
         int64_t r[4];
