@@ -120,6 +120,11 @@ void zk_gemm_set_path(int path);
 int zk_gemm_get_path(void);
 /* What the last GEMM-like call used: path (1/2) and the limb counts of A and B (0 for the VALU path). */
 void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
+/* The MFMA path guesses how many base-256 digits the operands need and checks the guess on the device.  A call
+ * whose operands (pointer, shape) were seen before does not wait for that check: a guarded vector-ALU launch
+ * behind it recomputes the outputs if the guess was too small.  This returns how many calls so far needed that
+ * recomputation (counted once their ranges have reached the host; it waits for nothing). */
+long zk_gemm_guard_hits(void);
 
 /* HIP-event stopwatch on the null stream (the stream every entry point launches on). */
 void zk_timer_start(void);

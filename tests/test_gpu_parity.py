@@ -397,17 +397,62 @@ def test_gemm_mfma_path_is_taken(K, oracle):
     A = rand_i64(rng, (1, 64, 256), 20)
     W = rand_i64(rng, (128, 256), 16)
     K.lib.zk_gemm_set_path(2)
-    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    dA, dW = dev(A), dev(W)
+    C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
     assert K.gemm_last_plan() == (2, 3, 3)
     Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 29)
     assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
     A = rand_i64(rng, (1, 64, 256), 63)
     W = rand_i64(rng, (128, 256), 63)
-    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    dA2, dW2 = dev(A), dev(W)            # the first pair stays alive: new addresses, nothing remembered about them
+    C, R = K.int64_bmm_broadcast(dA2, dW2, 1, 1, 29)
     assert K.gemm_last_plan() == (2, 9, 9)
     K.lib.zk_gemm_set_path(1)
-    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29)
+    C, R = K.int64_bmm_broadcast(dA2, dW2, 1, 1, 29)
     assert K.gemm_last_plan() == (1, 0, 0)
+    K.lib.zk_gemm_set_path(0)
+
+
+@pytest.mark.parametrize("M", [16, 48])
+def test_gemm_stale_digit_guess_is_caught(K, oracle, M):
+    """Operands that change in place under the same pointers.  The call after the change runs on the digit
+    counts remembered for those pointers and does not wait for their check; the guarded recomputation behind
+    it must still deliver exact results, and the following call must have learnt the new range."""
+    rng = np.random.default_rng(7 + M)
+    A = rand_i64(rng, (1, M, 512), 20)
+    W = rand_i64(rng, (160, 512), 16)
+    dA, dW = dev(A), dev(W)
+    K.lib.zk_gemm_set_path(2)
+    for _ in range(2):
+        C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
+        assert K.gemm_last_plan() == (2, 3, 3)
+    Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 29)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    hits = K.lib.zk_gemm_guard_hits()
+
+    A2 = rand_i64(rng, A.shape, 63)
+    W2 = rand_i64(rng, W.shape, 40)
+    dA.copy_(torch.from_numpy(A2))
+    dW.copy_(torch.from_numpy(W2))
+    C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
+    assert K.gemm_last_plan() == (2, 3, 3), "this call is expected to run on the stale guess"
+    Ce, Re = oracle.int64_bmm_broadcast(A2, W2, 1, 1, 29)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    assert K.lib.zk_gemm_guard_hits() == hits + 1
+    C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
+    assert K.gemm_last_plan()[0] == 2 and K.gemm_last_plan()[1] == 9 and K.gemm_last_plan()[2] >= 6
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    assert K.lib.zk_gemm_guard_hits() == hits + 1
+
+    # and back: one call on digit counts that are wider than needed, then the narrow ones again
+    dA.copy_(torch.from_numpy(A))
+    dW.copy_(torch.from_numpy(W))
+    Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 29)
+    C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 29)
+    assert K.gemm_last_plan() == (2, 3, 3)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
     K.lib.zk_gemm_set_path(0)
 
 

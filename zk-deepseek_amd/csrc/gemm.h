@@ -26,12 +26,17 @@ struct GemmDesc {
 
 enum GemmPath { kPathAuto = 0, kPathValu = 1, kPathMfma = 2 };
 
-// Native 64-bit multiply-add chains on the vector ALU; handles every descriptor.
-void gemm_valu_launch(const GemmDesc &d);
+// Native 64-bit multiply-add chains on the vector ALU; handles every descriptor.  With a `guard` (device
+// pointer) the launch is conditional: its workgroups return at once unless *guard is non-zero when they start.
+void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard = nullptr);
 
 // Limb-decomposed i8 MFMA.  Returns false (nothing launched) when the descriptor is outside what it
 // supports, in which case the caller falls back to the VALU path.
 bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
+
+// Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
+// vector-ALU recomputation (known once their range has reached the host).
+long gemm_mfma_guard_hits();
 
 // Top-level dispatch used by the extern "C" launchers.
 void gemm_dispatch(const char *name, const GemmDesc &d);

@@ -152,4 +152,6 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b)
     if (limbs_b) *limbs_b = zk::g_last_lb;
 }
 
+long zk_gemm_guard_hits(void) { return zk::gemm_mfma_guard_hits(); }
+
 }  // extern "C"

@@ -17,15 +17,21 @@
 // RUN*OCTS apart.  Adjacent lanes then read adjacent 16-byte pieces and every 64-byte line of the tile is
 // fetched by exactly one load instruction.
 //
-// The digit counts are speculated from a cached or sampled range; the workgroups of the first tile row /
-// column track the exact min and max of everything they load, the launcher reads them back and reruns with
-// wider digits in the rare case the guess was too small.  Results never depend on the guess.
+// The digit counts are speculated from a cached or sampled range.  The kernels track the exact min and max of
+// everything they load (every workgroup leaves its share in a slot of its own, a one-workgroup kernel folds
+// them and compares with the digit counts used).  The first call for an operand reads the verdict back and
+// reruns with wider digits if the guess was too small.  Later calls do not wait: a guarded launch of the
+// vector-ALU kernel follows, which recomputes everything if the verdict is bad and returns at once otherwise,
+// and the exact range travels to the host behind the stream to refresh the cache.  Results never depend on
+// the guess, and a call whose operands were seen before never blocks the host.
 #include "gemm.h"
+#include "../../include/int64gemm.h"
 
 #include <map>
 #include <mutex>
 #include <set>
 #include <tuple>
+#include <vector>
 #include <type_traits>
 
 // Tuning knobs: MFMA depths (32 k each) per pipeline step by diagonal count, and how many vector-ALU
@@ -56,7 +62,8 @@ struct MfmaParams {
     int M, N, K, shift;
     int64_t init;
     int tiles_m, tiles_n;
-    unsigned long long *range;      // [minA, maxA, minB, maxB], order-preserving unsigned images of int64
+    unsigned long long *range;      // [minA, maxA, minB, maxB], order-preserving unsigned images of int64; [4] verdict
+    unsigned long long *wg_range;   // one such quadruple per workgroup of the GEMM kernel
     int verify_b_all_batches;       // B differs per batch: every batch's first tile row tracks its range
     const unsigned char *a_planes;  // pre-split digits of A (planes variants only)
     int a_msub, a_ksteps;           // 32-row groups and 32-k steps the planes were written for
@@ -64,7 +71,11 @@ struct MfmaParams {
     // each cover a slice of K and leave raw 128-bit partial sums in `partials`
     int main_tiles, split;
     unsigned long long *partials;
+    int part64;                     // the partial sums fit 64 bits: only the low words are kept
     int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
+#ifdef ZK_DBG_TIMES
+    unsigned long long *dbg;
+#endif
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -121,8 +132,9 @@ __device__ __forceinline__ void limb_split8(const int64_t (&x)[8], uint2 (&out)[
 }
 
 // Smallest digit count whose range holds every value in [lo, hi].
-static int limbs_needed(int64_t lo, int64_t hi)
+__host__ __device__ static inline int limbs_needed(int64_t lo, int64_t hi)
 {
+    if (lo > hi) return 1;                   // nothing was seen
     for (int n = 1; n <= 8; n++) {
         // x + bias_n in [-2^(8n-1), 2^(8n-1))
         i128 bias = n == 1 ? 0 : (i128)(0x0080808080808080ull >> (8 * (8 - n)));
@@ -141,6 +153,12 @@ __device__ __forceinline__ void mm_update(MinMax &r, int64_t v)
     r.hi = v > r.hi ? v : r.hi;
 }
 
+__device__ __forceinline__ void mm_merge(MinMax &r, const MinMax &o)
+{
+    r.lo = o.lo < r.lo ? o.lo : r.lo;
+    r.hi = o.hi > r.hi ? o.hi : r.hi;
+}
+
 __device__ __forceinline__ MinMax mm_wave(MinMax r)
 {
 #pragma unroll
@@ -150,16 +168,6 @@ __device__ __forceinline__ MinMax mm_wave(MinMax r)
         r.hi = oh > r.hi ? oh : r.hi;
     }
     return r;
-}
-
-// single-lane publish of an already reduced range
-__device__ __forceinline__ void mm_publish_lane(MinMax r, unsigned long long *slot)
-{
-    const unsigned long long lo = (unsigned long long)r.lo ^ kSignFlip, hi = (unsigned long long)r.hi ^ kSignFlip;
-    if (r.lo <= r.hi) {
-        if (lo < __atomic_load_n(slot, __ATOMIC_RELAXED)) atomicMin(slot, lo);
-        if (hi > __atomic_load_n(slot + 1, __ATOMIC_RELAXED)) atomicMax(slot + 1, hi);
-    }
 }
 
 __device__ __forceinline__ void mm_publish(MinMax r, unsigned long long *slot)
@@ -295,38 +303,66 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
     __syncthreads();
     if (tid == 0) {
 #pragma unroll
-        for (int w = 1; w < 4; w++) { mm_update(r, red[w].lo); mm_update(r, red[w].hi); }
+        for (int w = 1; w < 4; w++) mm_merge(r, red[w]);
         const long b = ((long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
         mm[2 * b] = (unsigned long long)r.lo ^ kSignFlip;
         mm[2 * b + 1] = (unsigned long long)r.hi ^ kSignFlip;
     }
 }
 
-// Folds the per-workgroup ranges of the pre-pass into range[0..1] and resets the B slots range[2..3].
-__global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long long *mm, long count, unsigned long long *range)
+// Folds the per-workgroup ranges of the plane pre-pass (`mm`, A only) and of the GEMM kernel (`wg`, A and B) into
+// range[0..3] and leaves the verdict in range[4]: 0 when `na` and `nb` digits covered them, 1 otherwise.
+// `host_copy`, when set, is pinned host memory that receives the same five words.
+__global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long long *mm, long mm_count,
+                                                         const unsigned long long *wg, long wg_count,
+                                                         unsigned long long *range, int na, int nb,
+                                                         unsigned long long *host_copy)
 {
-    __shared__ unsigned long long lo_s[4], hi_s[4];
-    unsigned long long lo = ~0ull, hi = 0ull;
-    for (long i = threadIdx.x; i < count; i += 256) {
+    __shared__ unsigned long long red[4][4];
+    unsigned long long v[4] = { ~0ull, 0ull, ~0ull, 0ull };
+    for (long i = threadIdx.x; i < mm_count; i += 256) {
         const unsigned long long a = mm[2 * i], b = mm[2 * i + 1];
-        lo = a < lo ? a : lo;
-        hi = b > hi ? b : hi;
+        v[0] = a < v[0] ? a : v[0];
+        v[1] = b > v[1] ? b : v[1];
+    }
+    for (long i = threadIdx.x; i < wg_count; i += 256) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const unsigned long long a = wg[4 * i + q];
+            v[q] = (q & 1) ? (a > v[q] ? a : v[q]) : (a < v[q] ? a : v[q]);
+        }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const unsigned long long ol = (unsigned long long)__shfl_xor((long long)lo, off, kWave);
-        const unsigned long long oh = (unsigned long long)__shfl_xor((long long)hi, off, kWave);
-        lo = ol < lo ? ol : lo;
-        hi = oh > hi ? oh : hi;
+    for (int q = 0; q < 4; q++) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const unsigned long long o = (unsigned long long)__shfl_xor((long long)v[q], off, kWave);
+            v[q] = (q & 1) ? (o > v[q] ? o : v[q]) : (o < v[q] ? o : v[q]);
+        }
     }
-    if ((threadIdx.x & 63) == 0) { lo_s[threadIdx.x >> 6] = lo; hi_s[threadIdx.x >> 6] = hi; }
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) red[threadIdx.x >> 6][q] = v[q];
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < 4; i++) { lo = lo_s[i] < lo ? lo_s[i] : lo; hi = hi_s[i] > hi ? hi_s[i] : hi; }
-        range[0] = lo;
-        range[1] = hi;
-        range[2] = ~0ull;
-        range[3] = 0ull;
+        for (int w = 1; w < 4; w++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const unsigned long long o = red[w][q];
+                v[q] = (q & 1) ? (o > v[q] ? o : v[q]) : (o < v[q] ? o : v[q]);
+            }
+#pragma unroll
+        for (int q = 0; q < 4; q++) range[q] = v[q];
+        const int need_a = limbs_needed((int64_t)(v[0] ^ kSignFlip), (int64_t)(v[1] ^ kSignFlip));
+        const int need_b = limbs_needed((int64_t)(v[2] ^ kSignFlip), (int64_t)(v[3] ^ kSignFlip));
+        const unsigned long long verdict = (need_a <= na && need_b <= nb) ? 0ull : 1ull;
+        range[4] = verdict;
+        if (host_copy) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) host_copy[q] = v[q];
+            host_copy[4] = verdict;
+        }
     }
 }
 
@@ -352,6 +388,12 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WVN, wn = wave % WVN;
+#ifdef ZK_DBG_TIMES
+#define ZK_STAMP(i) do { if (tid == 0) p.dbg[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define ZK_STAMP(i)
+#endif
+    ZK_STAMP(0);
 
     // workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of them, each with its own L2), so
     // ids are regrouped to give each XCD a contiguous run of tiles; within a run the tile-row index moves
@@ -647,13 +689,16 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         if (ks_begin + 1 < full_steps) fetch(ks_begin + 1, std::true_type()); else fetch(ks_begin + 1, std::false_type());
     }
     __syncthreads();
+    ZK_STAMP(1);
     int ks = ks_begin;
     const int fast_end = full_steps < ks_end ? full_steps : ks_end;
     for (; ks + 2 < fast_end; ks++) step_body(ks, std::true_type());
     for (; ks + 1 < ks_end; ks++) step_body(ks, std::false_type());
     compute_all((ks_end - 1 - ks_begin) & 1);
+    ZK_STAMP(2);
 
-    // one publishing lane per workgroup: the waves' ranges meet in LDS (the stages are free by now)
+    // every workgroup leaves its ranges (empty ones included) in its own slot; the waves' ranges meet in LDS
+    // (the stages are free by now)
     if (verify_a || verify_b) {
         __syncthreads();
         MinMax *red = reinterpret_cast<MinMax *>(smem);
@@ -662,14 +707,17 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         if (lane == 0) { red[2 * wave] = ra; red[2 * wave + 1] = rb; }
         __syncthreads();
         if (tid == 0) {
-            for (int w = 1; w < T / 64; w++) {
-                mm_update(ra, red[2 * w].lo); mm_update(ra, red[2 * w].hi);
-                mm_update(rb, red[2 * w + 1].lo); mm_update(rb, red[2 * w + 1].hi);
-            }
-            if (verify_a) mm_publish_lane(ra, p.range);
-            if (verify_b) mm_publish_lane(rb, p.range + 2);
+            for (int w = 1; w < T / 64; w++) { mm_merge(ra, red[2 * w]); mm_merge(rb, red[2 * w + 1]); }
         }
     }
+    if (tid == 0) {
+        unsigned long long *slot = p.wg_range + 4 * (long)blockIdx.x;
+        slot[0] = (unsigned long long)ra.lo ^ kSignFlip;
+        slot[1] = (unsigned long long)ra.hi ^ kSignFlip;
+        slot[2] = (unsigned long long)rb.lo ^ kSignFlip;
+        slot[3] = (unsigned long long)rb.hi ^ kSignFlip;
+    }
+    ZK_STAMP(3);
     if (pf_acc == 0x7f3a91c5 && p.shift == 99) p.C[0] = pf_acc;      // never true: keeps the warm-up loads alive
 
     // epilogue: diagonals -> 128-bit sum -> shift.  Accumulator register r of lane l holds
@@ -683,6 +731,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                // rows of this register that all lie past M (uniform over the wave): nothing to keep
+                if (nsplit > 1 && m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= p.M) continue;
                 // whole tiles start from the rounding term; split workgroups leave it to the finishing kernel
                 uint64_t lo = nsplit > 1 ? 0 : (uint64_t)p.init, hi = nsplit > 1 ? 0 : (uint64_t)(p.init >> 63);
 #pragma unroll
@@ -698,11 +748,11 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                     lo = s;
                 }
                 if (nsplit > 1) {
-                    // raw partial sum (without init): 16 bytes per output, lane-contiguous, finished by
-                    // gemm_split_finish_kernel
-                    const long e = ((((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r) * 64 + lane;
-                    p.partials[2 * e] = lo;
-                    p.partials[2 * e + 1] = hi;
+                    // raw partial sum (without init), finished by gemm_split_finish_kernel: 64 lanes' low words, then
+                    // (unless 64 bits hold the sums) their high words, per (slice, wave, tile, register)
+                    const long q = (((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r;
+                    if (p.part64) p.partials[q * 64 + lane] = lo;
+                    else { p.partials[q * 128 + lane] = lo; p.partials[q * 128 + 64 + lane] = hi; }
                 } else if (m < p.M && n < p.N) {
                     const long o = (long)g * p.sC + (long)m * p.ldc + n;
                     uint64_t q;
@@ -714,6 +764,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             }
         }
     }
+    ZK_STAMP(4);
 }
 
 // Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
@@ -739,13 +790,26 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
             for (int r4 = 0; r4 < r_per; r4++) {
                 const int r = rq * r_per + r4;
                 const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= p.M) continue;      // never written
                 uint64_t lo = (uint64_t)p.init, hi = (uint64_t)(p.init >> 63);
-                for (int sidx = 0; sidx < p.split; sidx++) {
-                    const long e = ((((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r) * 64 + lane;
-                    const uint64_t plo = p.partials[2 * e], phi = p.partials[2 * e + 1];
-                    const uint64_t s = lo + plo;
-                    hi += phi + (s < lo ? 1 : 0);
-                    lo = s;
+                const long q0 = ((long)tail_tile * p.split * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r;
+                const long qs = (long)(T / 64) * (WM * WN * 16);          // from one slice to the next
+                if (p.part64) {
+                    uint64_t s = 0;
+#pragma unroll 8
+                    for (int sidx = 0; sidx < p.split; sidx++) s += p.partials[(q0 + sidx * qs) * 64 + lane];
+                    const uint64_t t = lo + s;
+                    hi += (uint64_t)((int64_t)s >> 63) + (t < lo ? 1 : 0);
+                    lo = t;
+                } else {
+#pragma unroll 4
+                    for (int sidx = 0; sidx < p.split; sidx++) {
+                        const uint64_t plo = p.partials[(q0 + sidx * qs) * 128 + lane];
+                        const uint64_t phi = p.partials[(q0 + sidx * qs) * 128 + 64 + lane];
+                        const uint64_t t = lo + plo;
+                        hi += phi + (t < lo ? 1 : 0);
+                        lo = t;
+                    }
                 }
                 if (m < p.M && n < p.N) {
                     const long o = (long)g * p.sC + (long)m * p.ldc + n;
@@ -840,36 +904,114 @@ static const Instance *pick_instance(int na, int nb, bool b32, bool skinny)
     return best;
 }
 
+typedef std::tuple<const void *, long, long, int> OperandKey;     // (pointer, rows, K, element size)
+
+// A range on its way from the device to the host behind the stream (calls that do not wait for their verdict).
+struct PendingRange {
+    hipEvent_t ev = nullptr;
+    unsigned long long *host = nullptr;      // pinned: [minA, maxA, minB, maxB, verdict]
+    OperandKey key_a, key_b;
+    bool busy = false;
+};
+
+constexpr int kPendingSlots = 16;
+
 struct RangeCache {
     std::mutex mu;
-    std::map<std::tuple<const void *, long, long, int>, int> limbs;     // (ptr, rows, K, elem size) -> digits
-    unsigned long long *dev = nullptr;       // [minA, maxA, minB, maxB]
+    std::map<OperandKey, int> limbs;         // operand -> digits its values needed when last seen
+    unsigned long long *dev = nullptr;       // [minA, maxA, minB, maxB, verdict]
     unsigned char *planes = nullptr;         // digit planes of A, grown on demand, kept for the process lifetime
     size_t planes_bytes = 0;
     unsigned long long *mm = nullptr;        // per-workgroup ranges of the plane pre-pass
     size_t mm_count = 0;
-    unsigned long long *partials = nullptr;  // 128-bit partial sums of split tail tiles
+    unsigned long long *wg = nullptr;        // per-workgroup ranges of the GEMM kernel
+    size_t wg_count = 0;
+    unsigned long long *partials = nullptr;  // partial sums of split tiles
     size_t partials_bytes = 0;
     int cus = 0;                             // compute units of the device
-    int lookup(const void *ptr, long rows, long K, int esz)
+    PendingRange pending[kPendingSlots];
+    unsigned long long *pinned = nullptr;
+    int pending_head = 0;                    // next slot to use; slots are used and drained in ring order
+    long guard_hits = 0;                     // calls whose speculation failed after they had returned
+    int lookup(const OperandKey &k)
     {
-        auto it = limbs.find(std::make_tuple(ptr, rows, K, esz));
+        auto it = limbs.find(k);
         return it == limbs.end() ? 0 : it->second;
     }
-    void store(const void *ptr, long rows, long K, int esz, int n)
+    void store(const OperandKey &k, int n)
     {
         if (limbs.size() > 4096) limbs.clear();
-        limbs[std::make_tuple(ptr, rows, K, esz)] = n;
+        limbs[k] = n;
     }
 };
 
 static RangeCache g_cache;
+
+// Grows a device buffer kept for the process lifetime.  Returns false (buffer left empty) when memory is short.
+template <typename T>
+static bool grow(T *&buf, size_t &have, size_t need, const char *what)
+{
+    if (need <= have) return true;
+    if (buf && hipFree(buf) != hipSuccess) { set_error(kLaunchFailure, "gemm: cannot release the %s", what); return false; }
+    buf = nullptr;
+    have = 0;
+    if (hipMalloc(&buf, need * sizeof(T)) != hipSuccess) { (void)hipGetLastError(); buf = nullptr; return false; }
+    have = need;
+    return true;
+}
 
 static bool read_range(unsigned long long *dev, int64_t (&out)[4])
 {
     unsigned long long h[4];
     if (hipMemcpy(h, dev, sizeof(h), hipMemcpyDeviceToHost) != hipSuccess) return false;
     for (int i = 0; i < 4; i++) out[i] = (int64_t)(h[i] ^ kSignFlip);
+    return true;
+}
+
+// Takes in the ranges that have arrived since the last call, oldest first.
+static void drain_pending()
+{
+    for (int n = 0; n < kPendingSlots; n++) {
+        PendingRange &s = g_cache.pending[(g_cache.pending_head + n) % kPendingSlots];
+        if (!s.busy) continue;
+        const hipError_t st = hipEventQuery(s.ev);
+        if (st != hipSuccess) { (void)hipGetLastError(); if (st == hipErrorNotReady) continue; }
+        if (st == hipSuccess) {
+            g_cache.store(s.key_a, limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip)));
+            g_cache.store(s.key_b, limbs_needed((int64_t)(s.host[2] ^ kSignFlip), (int64_t)(s.host[3] ^ kSignFlip)));
+            if (s.host[4]) g_cache.guard_hits++;
+        }
+        s.busy = false;
+    }
+}
+
+long gemm_mfma_guard_hits()
+{
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    drain_pending();
+    return g_cache.guard_hits;
+}
+
+static bool init_cache()
+{
+    if (g_cache.dev) return true;
+    if (hipMalloc(&g_cache.dev, 8 * sizeof(unsigned long long)) != hipSuccess) {
+        set_error(kLaunchFailure, "gemm: cannot allocate the 64-byte range buffer");
+        return false;
+    }
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    g_cache.cus = n;
+    // without the pinned slots every call simply waits for its own verdict
+    if (hipHostMalloc(&g_cache.pinned, kPendingSlots * 8 * sizeof(unsigned long long), hipHostMallocDefault) == hipSuccess) {
+        for (int i = 0; i < kPendingSlots; i++) {
+            g_cache.pending[i].host = g_cache.pinned + 8 * i;
+            if (hipEventCreateWithFlags(&g_cache.pending[i].ev, hipEventDisableTiming) != hipSuccess) g_cache.pending[i].ev = nullptr;
+        }
+    } else {
+        (void)hipGetLastError();
+        g_cache.pinned = nullptr;
+    }
     return true;
 }
 
@@ -880,12 +1022,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     if (d.G > 65535) return false;
     const bool kmajor = d.ldbn == 1 && d.ldbk != 1;
     std::lock_guard<std::mutex> lock(g_cache.mu);
-    if (!g_cache.dev) {
-        if (hipMalloc(&g_cache.dev, 4 * sizeof(unsigned long long)) != hipSuccess) {
-            set_error(kLaunchFailure, "gemm: cannot allocate the 32-byte range buffer");
-            return false;
-        }
-    }
+    if (!init_cache()) return false;
+    drain_pending();
 
     MfmaParams p;
     p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
@@ -893,18 +1031,17 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift; p.init = d.init;
     p.range = g_cache.dev;
     p.verify_b_all_batches = d.sB != 0;
-    p.a_planes = nullptr; p.a_msub = 0; p.a_ksteps = 0;
-    p.main_tiles = 0; p.split = 1; p.partials = nullptr; p.finish_rq = 4;
-    if (!g_cache.cus) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        g_cache.cus = n;
-    }
 
-    const long rows_a = (long)d.G * d.M;
-    int na = g_cache.lookup(d.A, rows_a, d.K, 8);
-    int nb = g_cache.lookup(d.B, d.N, d.K, d.b32 ? 4 : 8);
+    const OperandKey key_a(d.A, (long)d.G * d.M, d.K, 8), key_b(d.B, d.N, d.K, d.b32 ? 4 : 8);
+    int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
+    // Operands seen before: speculate, do not wait.  Otherwise sample them and check the verdict before returning.
+    PendingRange *slot = nullptr;
+    if (na && nb && g_cache.pinned && getenv("ZK_GEMM_SYNC") == nullptr) {
+        PendingRange &s = g_cache.pending[g_cache.pending_head];
+        if (!s.busy && s.ev) slot = &s;
+    }
     if (!na || !nb) {
+        p.tiles_m = p.tiles_n = 1;
         range_reset_kernel<<<1, 64, 0, 0>>>(p.range);
         range_sample_kernel<<<1, 256, 0, 0>>>(p, d.b32, d.G, 0);
         range_sample_kernel<<<1, 256, 0, 0>>>(p, d.b32, d.G, 1);
@@ -927,68 +1064,24 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         p.tiles_n = (d.N + BN - 1) / BN;
         const long per_batch = (long)p.tiles_m * p.tiles_n;
         if (per_batch > 0x7FFFFFFFL) return false;
+        const long total = per_batch * d.G;
+        if (total > 0x7FFFFFFFL / 8) return false;
         // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass
         const bool use_planes = !kmajor && p.tiles_n >= 4;
         const int variant = kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
         if (!fn) return false;
-        if (!use_planes) range_reset_kernel<<<1, 64, 0, 0>>>(p.range);       // with planes the fold kernel does it
-        if (use_planes) {
-            const int msub = p.tiles_m * (BM / 32);
-            const size_t need = (size_t)d.G * msub * ksteps * inst->na * 1024;
-            if (need > g_cache.planes_bytes) {
-                if (g_cache.planes && hipFree(g_cache.planes) != hipSuccess) {
-                    set_error(kLaunchFailure, "gemm: cannot release the digit-plane buffer");
-                    return false;
-                }
-                g_cache.planes = nullptr;
-                g_cache.planes_bytes = 0;
-                if (hipMalloc(&g_cache.planes, need) != hipSuccess) {
-                    (void)hipGetLastError();
-                    return false;                    // not enough memory for planes: the caller uses the VALU path
-                }
-                g_cache.planes_bytes = need;
-            }
-            p.a_planes = g_cache.planes; p.a_msub = msub; p.a_ksteps = ksteps;
-            const int rows_per_wg = 256 / (4 * inst->kk);
-            const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)(msub * 32 / rows_per_wg), (unsigned)d.G);
-            const size_t wgs = (size_t)pgrid.x * pgrid.y * pgrid.z;
-            if (wgs > g_cache.mm_count) {
-                if (g_cache.mm && hipFree(g_cache.mm) != hipSuccess) {
-                    set_error(kLaunchFailure, "gemm: cannot release the range scratch");
-                    return false;
-                }
-                g_cache.mm = nullptr;
-                g_cache.mm_count = 0;
-                if (hipMalloc(&g_cache.mm, wgs * 2 * sizeof(unsigned long long)) != hipSuccess) {
-                    (void)hipGetLastError();
-                    return false;
-                }
-                g_cache.mm_count = wgs;
-            }
-            inst->planes[d.b32 ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
-            range_fold_kernel<<<1, 256, 0, 0>>>(g_cache.mm, (long)wgs, p.range);
-        }
-        const size_t lds = 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
-        static std::set<const void *> lds_raised;
-        if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
-            if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-                set_error(kLaunchFailure, "gemm: cannot raise the LDS limit to %zu bytes", lds);
-                return false;
-            }
-            lds_raised.insert((const void *)fn);
-        }
-        // Tail split: with `total` tiles on `cus` compute units the last partial round would leave most of the
-        // device idle.  Its tiles are cut into `split` slices of K each, run as extra workgroups in the same
-        // launch, and a small kernel adds the 128-bit partial sums.
-        const long total = per_batch * d.G;
-        if (total > 0x7FFFFFFFL / 8) return false;
-        // A launch smaller than the device is split the same way over all of its tiles.
+
+        // Split-K: a launch smaller than the device is cut into `split` slices of K per tile, each a workgroup of
+        // its own; with more tiles than compute units the same is done for the tiles of the last, partial round
+        // only.  The slices leave raw partial sums and a small kernel adds them.
         const int steps = (d.K + 32 * inst->kk - 1) / (32 * inst->kk);
         int tail = (int)(total % g_cache.cus), split = 1;
         p.main_tiles = (int)total;
         p.split = 1;
+        p.partials = nullptr;
+        p.part64 = 0;
         p.finish_rq = 4;
         if (getenv("ZK_NO_TAIL_SPLIT") == nullptr) {
             if (total < g_cache.cus) {
@@ -1004,37 +1097,92 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             }
         }
         if (split >= 2) {
-            const size_t need = (size_t)tail * split * BM * BN * 16;
-            if (need > g_cache.partials_bytes) {
-                if (g_cache.partials && hipFree(g_cache.partials) != hipSuccess) {
-                    set_error(kLaunchFailure, "gemm: cannot release the partial-sum buffer");
-                    return false;
-                }
-                g_cache.partials = nullptr;
-                g_cache.partials_bytes = 0;
-                if (hipMalloc(&g_cache.partials, need) == hipSuccess) g_cache.partials_bytes = need;
-                else (void)hipGetLastError();
-            }
-            if (g_cache.partials) {
+            // |sum| < K * 2^(8(NA+NB)-2): below 2^62 the low word alone carries a partial sum
+            int kbits = 0;
+            while ((1L << kbits) < (long)ksteps * 32) kbits++;
+            const bool part64 = 8 * (inst->na + inst->nb) - 2 + kbits <= 62;
+            const size_t need = (size_t)tail * split * BM * BN * (part64 ? 1 : 2);
+            if (grow(g_cache.partials, g_cache.partials_bytes, need, "partial-sum buffer")) {
                 p.main_tiles = (int)(total - tail);
                 p.split = split;
                 p.partials = g_cache.partials;
-            }
+                p.part64 = part64 ? 1 : 0;
+            } else if (zk_last_error() != kOk) return false;
         }
         const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
+        if (!grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return false;
+        p.wg_range = g_cache.wg;
+
+        long plane_wgs = 0;
+        p.a_planes = nullptr; p.a_msub = 0; p.a_ksteps = 0;
+        if (use_planes) {
+            const int msub = p.tiles_m * (BM / 32);
+            const size_t need = (size_t)d.G * msub * ksteps * inst->na * 1024;
+            // not enough memory for planes: the caller uses the VALU path
+            if (!grow(g_cache.planes, g_cache.planes_bytes, need, "digit-plane buffer")) return false;
+            p.a_planes = g_cache.planes; p.a_msub = msub; p.a_ksteps = ksteps;
+            const int rows_per_wg = 256 / (4 * inst->kk);
+            const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)(msub * 32 / rows_per_wg), (unsigned)d.G);
+            plane_wgs = (long)pgrid.x * pgrid.y * pgrid.z;
+            if (!grow(g_cache.mm, g_cache.mm_count, (size_t)plane_wgs * 2, "range scratch")) return false;
+            inst->planes[d.b32 ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
+        }
+        const size_t lds = 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
+        static std::set<const void *> lds_raised;
+        if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
+            if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+                set_error(kLaunchFailure, "gemm: cannot raise the LDS limit to %zu bytes", lds);
+                return false;
+            }
+            lds_raised.insert((const void *)fn);
+        }
+#ifdef ZK_DBG_TIMES
+        static unsigned long long *dbg_dev = nullptr;
+        if (!dbg_dev) (void)hipMalloc(&dbg_dev, 8 * 8 * 65536);
+        p.dbg = dbg_dev;
+#endif
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
+#ifdef ZK_DBG_TIMES
+        if (getenv("ZK_DBG_DUMP")) {
+            std::vector<unsigned long long> h(blocks * 8);
+            (void)hipMemcpy(h.data(), dbg_dev, blocks * 64, hipMemcpyDeviceToHost);
+            unsigned long long t0 = ~0ull;
+            for (long b = 0; b < blocks; b++) t0 = h[b * 8] < t0 ? h[b * 8] : t0;
+            double avg[5] = {0}, mx[5] = {0};
+            for (long b = 0; b < blocks; b++)
+                for (int i = 0; i < 5; i++) { double v = (double)(h[b * 8 + i] - t0) * 0.01; avg[i] += v / blocks; mx[i] = v > mx[i] ? v : mx[i]; }
+            fprintf(stderr, "dbg times us (avg/max since first start) blocks=%ld:", blocks);
+            for (int i = 0; i < 5; i++) fprintf(stderr, " [%d] %.2f/%.2f", i, avg[i], mx[i]);
+            fprintf(stderr, "\n");
+        }
+#endif
         if (p.split > 1) {
             inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq)), dim3((unsigned)inst->threads), 0, 0>>>(p);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
         }
+        range_fold_kernel<<<1, 256, 0, 0>>>(g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb,
+                                            slot ? slot->host : nullptr);
+        *limbs_a = inst->na;
+        *limbs_b = inst->nb;
+        if (slot) {
+            // no waiting: the vector-ALU kernel redoes the product if the verdict is bad, the range follows later
+            gemm_valu_launch(d, p.range + 4);
+            if (hipEventRecord(slot->ev, 0) == hipSuccess) {
+                slot->key_a = key_a;
+                slot->key_b = key_b;
+                slot->busy = true;
+                g_cache.pending_head = (g_cache.pending_head + 1) % kPendingSlots;
+            } else {
+                (void)hipGetLastError();
+            }
+            return true;
+        }
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
-        g_cache.store(d.A, rows_a, d.K, 8, need_a);
-        g_cache.store(d.B, d.N, d.K, d.b32 ? 4 : 8, need_b);
-        *limbs_a = inst->na;
-        *limbs_b = inst->nb;
+        g_cache.store(key_a, need_a);
+        g_cache.store(key_b, need_b);
         if (need_a <= inst->na && need_b <= inst->nb) return true;
         na = need_a;
         nb = need_b;

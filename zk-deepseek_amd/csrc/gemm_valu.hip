@@ -5,6 +5,9 @@
 // tiles of 16 k-steps are staged through LDS transposed to [k][row] so the inner loop reads 32-byte
 // vectors; global loads are 128-byte row segments.  Handles every descriptor: int32 or int64 B, either B
 // layout, operand divisors, any shape.
+//
+// The same kernel is the safety net of the speculating MFMA path: launched with a `guard` word, its workgroups
+// return at once unless that word says the speculation failed, in which case they recompute every output.
 #include "gemm.h"
 
 namespace zk {
@@ -20,6 +23,9 @@ struct ValuParams {
     long lda, sA, ldbn, ldbk, sB, ldc, sC;
     int M, N, K, shift;
     int64_t init, a_rs, b_rs;
+    int tiles_m, tiles_n;
+    long tiles;                               // tiles_m * tiles_n * G, walked by a 1-D grid
+    const unsigned long long *guard;          // when set: do nothing unless *guard != 0
 };
 
 template <bool B32>
@@ -35,8 +41,11 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(ValuParams p)
     __shared__ int64_t Bs[kVK][kVP];
 
     const int tid = threadIdx.x;
-    const int g = blockIdx.z;
-    const int m0 = blockIdx.y * kVT, n0 = blockIdx.x * kVT;
+    if (p.guard && __atomic_load_n(p.guard, __ATOMIC_RELAXED) == 0) return;
+    for (long tile = blockIdx.x; tile < p.tiles; tile += gridDim.x) {
+    const int g = (int)(tile / ((long)p.tiles_m * p.tiles_n));
+    const int rem = (int)(tile - (long)g * p.tiles_m * p.tiles_n);
+    const int m0 = (rem / p.tiles_n) * kVT, n0 = (rem % p.tiles_n) * kVT;
     const int64_t *Ag = p.A + (long)g * p.sA;
     const long boff = (long)g * p.sB;
 
@@ -108,6 +117,7 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(ValuParams p)
             if (p.R) p.R[o] = (int64_t)((uint64_t)sum & rmask);
         }
     }
+    }
 }
 
 template <bool B32, bool KMAJOR>
@@ -117,34 +127,24 @@ static void launch2(const ValuParams &p, dim3 grid, bool rescale)
     else gemm_valu_kernel<B32, KMAJOR, false><<<grid, dim3(256), 0, 0>>>(p);
 }
 
-void gemm_valu_launch(const GemmDesc &d)
+void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard)
 {
     ValuParams p;
     p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
     p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift;
     p.init = d.init; p.a_rs = d.a_rs; p.b_rs = d.b_rs;
+    p.tiles_m = (d.M + kVT - 1) / kVT;
+    p.tiles_n = (d.N + kVT - 1) / kVT;
+    p.tiles = (long)p.tiles_m * p.tiles_n * d.G;
+    p.guard = guard;
     const bool rescale = d.a_rs != 1 || d.b_rs != 1;
     const bool kmajor = d.ldbn == 1 && d.ldbk != 1;
-    const int gy_total = (d.M + kVT - 1) / kVT;
-    const int gx = (d.N + kVT - 1) / kVT;
-    // grid.y and grid.z are limited to 65535: walk M and G in chunks when they are larger
-    for (int g0 = 0; g0 < d.G; g0 += 65535) {
-        int gz = d.G - g0 < 65535 ? d.G - g0 : 65535;
-        for (int y0 = 0; y0 < gy_total; y0 += 65535) {
-            int gy = gy_total - y0 < 65535 ? gy_total - y0 : 65535;
-            ValuParams q = p;
-            q.A = p.A + (long)g0 * p.sA + (long)y0 * kVT * p.lda;
-            q.B = d.b32 ? (const void *)((const int32_t *)p.B + (long)g0 * p.sB)
-                        : (const void *)((const int64_t *)p.B + (long)g0 * p.sB);
-            q.C = p.C + (long)g0 * p.sC + (long)y0 * kVT * p.ldc;
-            q.R = p.R ? p.R + (long)g0 * p.sC + (long)y0 * kVT * p.ldc : nullptr;
-            q.M = d.M - y0 * kVT;
-            dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)gz);
-            if (d.b32) { if (kmajor) launch2<true, true>(q, grid, rescale); else launch2<true, false>(q, grid, rescale); }
-            else { if (kmajor) launch2<false, true>(q, grid, rescale); else launch2<false, false>(q, grid, rescale); }
-        }
-    }
+    // a guarded launch normally finds nothing to do, so it is kept small; either way workgroups stride over the tiles
+    const long cap = guard ? 2048 : (1L << 22);
+    dim3 grid((unsigned)(p.tiles < cap ? p.tiles : cap));
+    if (d.b32) { if (kmajor) launch2<true, true>(p, grid, rescale); else launch2<true, false>(p, grid, rescale); }
+    else { if (kmajor) launch2<false, true>(p, grid, rescale); else launch2<false, false>(p, grid, rescale); }
 }
 
 }  // namespace zk

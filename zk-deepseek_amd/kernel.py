@@ -64,6 +64,7 @@ lib.zk_gemm_set_path.argtypes = [_ci]
 lib.zk_gemm_get_path.restype = _ci
 lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
 lib.zk_timer_stop_ms.restype = ctypes.c_float
+lib.zk_gemm_guard_hits.restype = ctypes.c_long
 
 
 def _check(what):
