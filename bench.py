@@ -128,10 +128,20 @@ def main():
         pairs = la * lb
         ops = 2.0 * pairs * macs                         # i8 multiply-adds issued as MFMA, counted as 2 ops
         achieved = ops / (kern_ms * 1e-3) / 1e12
+        # what the i8 matrix pipe sustains on this box, measured live: register-resident and GEMM-shaped (fragments
+        # from LDS + a barrier per step), with zero operands and with random bytes.  The device is power managed
+        # and MFMAs on randomly toggling bytes (which the digits of real operands are) run slower than on zeros.
+        probe = {}
+        for name, with_lds, rnd in (("regs_zeros", 0, 0), ("regs_random", 0, 1), ("lds_zeros", 1, 0), ("lds_random", 1, 1)):
+            probe[name] = K.lib.zk_probe_mfma_i8_tops(with_lds, rnd, 3000)
+        K._check("MFMA probe")
         roofline = {"bound": "mfma", "achieved": achieved, "peak": I8_MFMA_PEAK_TOPS, "unit": "TOP/s",
                     "frac": achieved / I8_MFMA_PEAK_TOPS, "traffic": measured_traffic(),
+                    "path_peak_measured": probe,
+                    "frac_of_measured_random_data_peak": achieved / probe["regs_random"] if probe["regs_random"] else None,
                     "note": "i8 MFMA ops = 2 * limbs_a * limbs_b * M*N*K (%dx%d limb pairs per int64 MAC); "
-                            "duration = HIP events over the whole launcher" % (la, lb)}
+                            "duration = HIP events over the whole launcher; path_peak_measured = "
+                            "v_mfma_i32_32x32x32_i8 microbenchmark on this device, TOP/s" % (la, lb)}
     else:
         achieved = macs / (kern_ms * 1e-3) / 1e12
         roofline = {"bound": "valu", "achieved": achieved, "peak": None, "unit": "Tmac/s", "frac": None,

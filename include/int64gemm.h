@@ -126,6 +126,14 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
  * recomputation (counted once their ranges have reached the host; it waits for nothing). */
 long zk_gemm_guard_hits(void);
 
+/* Measurement helper for the roofline of the MFMA GEMM path: the sustained rate, in 10^12 i8 operations per
+ * second (2 per multiply-add), of a stream of v_mfma_i32_32x32x32_i8 shaped like the GEMM's inner loop (8 waves
+ * per compute unit, 10 accumulator tiles per wave).  with_lds: operand fragments re-read from LDS and a
+ * barrier per step, as in the GEMM; otherwise register resident.  random_data: operands are random bytes
+ * instead of zeros (the device is power managed and the rate depends on how the operand bits toggle).
+ * Allocates 4 bytes for the duration of the call and waits for its kernels. */
+double zk_probe_mfma_i8_tops(int with_lds, int random_data, int steps);
+
 /* HIP-event stopwatch on the null stream (the stream every entry point launches on). */
 void zk_timer_start(void);
 float zk_timer_stop_ms(void);   /* records the stop event, waits for it, returns elapsed milliseconds */

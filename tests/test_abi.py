@@ -35,7 +35,7 @@ def lib():
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return re.findall(r"^\s*(?:const\s+)?(?:void|int|long|float|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    return re.findall(r"^\s*(?:const\s+)?(?:void|int|long|float|double|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
 
 
 def test_header_declares_reference_abi():

@@ -31,19 +31,12 @@
 #include <mutex>
 #include <set>
 #include <tuple>
-#include <vector>
 #include <type_traits>
 
 // Tuning knobs: MFMA depths (32 k each) per pipeline step by diagonal count, and how many vector-ALU
 // instructions of the digit split are scheduled behind each MFMA of a step's last depth.
 #ifndef ZK_VALU_PER_MFMA
 #define ZK_VALU_PER_MFMA 8
-#endif
-#ifndef ZK_PREFETCH
-#define ZK_PREFETCH 0
-#endif
-#ifndef ZK_NARROW_LAYOUT
-#define ZK_NARROW_LAYOUT 0
 #endif
 #ifndef ZK_KK
 #define ZK_KK(DD) 1
@@ -73,9 +66,6 @@ struct MfmaParams {
     unsigned long long *partials;
     int part64;                     // the partial sums fit 64 bits: only the low words are kept
     int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
-#ifdef ZK_DBG_TIMES
-    unsigned long long *dbg;
-#endif
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -388,12 +378,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WVN, wn = wave % WVN;
-#ifdef ZK_DBG_TIMES
-#define ZK_STAMP(i) do { if (tid == 0) p.dbg[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define ZK_STAMP(i)
-#endif
-    ZK_STAMP(0);
 
     // workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of them, each with its own L2), so
     // ids are regrouped to give each XCD a contiguous run of tiles; within a run the tile-row index moves
@@ -494,35 +478,9 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         b_stride[it] = live ? STAGE : 0;
     }
 
-    // L2 warm-up: one dword from every 64-byte line of the B tile ZK_PREFETCH steps ahead of the staged loads.  The
-    // value only feeds a store that never happens; being issued after the real loads, it never delays their wait.
-    constexpr int B_STEP_BYTES = BK * (B32 ? 4 : 8);
-    constexpr int LINES_PER_ROW = B_STEP_BYTES / 64 > 0 ? B_STEP_BYTES / 64 : 1;
-    constexpr int PF_IT = (BKM || ZK_PREFETCH == 0) ? 0 : (BN * LINES_PER_ROW + T - 1) / T;
-    const char *pf_src[PF_IT > 0 ? PF_IT : 1];
-    int pf_acc = 0, pf_val[PF_IT > 0 ? PF_IT : 1] = { 0 };
-#pragma unroll
-    for (int it = 0; it < PF_IT; it++) {
-        const int l = it * T + tid;
-        int n = n0 + (l / LINES_PER_ROW) % BN;
-        n = n < p.N ? n : p.N - 1;
-        pf_src[it] = reinterpret_cast<const char *>(p.B) + ((long)g * p.sB + (long)n * p.ldbn) * (B32 ? 4 : 8) +
-                     (l % LINES_PER_ROW) * 64;
-    }
-    auto prefetch = [&](int ks) {
-#pragma unroll
-        for (int it = 0; it < PF_IT; it++) {
-            pf_acc |= pf_val[it];          // the value loaded one step ago: long since landed, no wait
-            pf_val[it] = *reinterpret_cast<const int *>(pf_src[it] + (long)ks * B_STEP_BYTES);
-        }
-    };
-
     // FAST: the whole step lies inside K and the pointers allow 16-byte loads: no guards at all.
     auto fetch = [&](int ks, auto fast_tag) {
         constexpr bool FAST = decltype(fast_tag)::value;
-#ifdef ZK_DBG_SAME_TILE
-        ks = FAST ? (ks & 1) : ks;
-#endif
         const int k0 = ks * BK;
         if (APL) {
 #pragma unroll
@@ -677,7 +635,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         __builtin_amdgcn_sched_barrier(0);
         track(ks + 1);
         if (ks + 2 < ks_end) fetch(ks + 2, fast_tag);
-        if (ZK_PREFETCH > 0 && decltype(fast_tag)::value && ks + 2 + ZK_PREFETCH < full_steps) prefetch(ks + 2 + ZK_PREFETCH);
         __syncthreads();
     };
 
@@ -689,13 +646,11 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         if (ks_begin + 1 < full_steps) fetch(ks_begin + 1, std::true_type()); else fetch(ks_begin + 1, std::false_type());
     }
     __syncthreads();
-    ZK_STAMP(1);
     int ks = ks_begin;
     const int fast_end = full_steps < ks_end ? full_steps : ks_end;
     for (; ks + 2 < fast_end; ks++) step_body(ks, std::true_type());
     for (; ks + 1 < ks_end; ks++) step_body(ks, std::false_type());
     compute_all((ks_end - 1 - ks_begin) & 1);
-    ZK_STAMP(2);
 
     // every workgroup leaves its ranges (empty ones included) in its own slot; the waves' ranges meet in LDS
     // (the stages are free by now)
@@ -717,8 +672,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         slot[2] = (unsigned long long)rb.lo ^ kSignFlip;
         slot[3] = (unsigned long long)rb.hi ^ kSignFlip;
     }
-    ZK_STAMP(3);
-    if (pf_acc == 0x7f3a91c5 && p.shift == 99) p.C[0] = pf_acc;      // never true: keeps the warm-up loads alive
 
     // epilogue: diagonals -> 128-bit sum -> shift.  Accumulator register r of lane l holds
     // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile.
@@ -764,7 +717,6 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             }
         }
     }
-    ZK_STAMP(4);
 }
 
 // Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
@@ -842,17 +794,10 @@ static Instance make_instance()
     static_assert(!SKINNY || DD <= 10, "skinny tiles keep two waves per SIMD");
     // narrow: 8 waves as 2x4, 64x32 per wave (128x128); mid: 8 waves as 4x2, 32x32 per wave (128x64);
     // wide: 4 waves as 2x2, 32x32 per wave (64x64, one wave per SIMD because of the accumulator count)
-#if 0
-    // narrow: 12 waves as 4x3, 32x32 per wave (128x96), three waves per SIMD
-    constexpr int WVM = DD <= 5 ? 4 : (DD <= 10 ? 4 : 2);
-    constexpr int WVN = DD <= 5 ? 3 : 2;
-    constexpr int WM = 1, WN = 1;
-#else
     // skinny (M <= 32): 8 waves as 1x8, 32x32 per wave (32x256)
     constexpr int WVM = SKINNY ? 1 : (DD <= 5 ? 2 : (DD <= 10 ? 4 : 2));
     constexpr int WVN = SKINNY ? 8 : (DD <= 5 ? 4 : 2);
     constexpr int WM = SKINNY ? 1 : (DD <= 5 ? 2 : 1), WN = 1;
-#endif
     constexpr int KK = ZK_KK(DD);
     Instance s;
     s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
@@ -1136,27 +1081,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             }
             lds_raised.insert((const void *)fn);
         }
-#ifdef ZK_DBG_TIMES
-        static unsigned long long *dbg_dev = nullptr;
-        if (!dbg_dev) (void)hipMalloc(&dbg_dev, 8 * 8 * 65536);
-        p.dbg = dbg_dev;
-#endif
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
-#ifdef ZK_DBG_TIMES
-        if (getenv("ZK_DBG_DUMP")) {
-            std::vector<unsigned long long> h(blocks * 8);
-            (void)hipMemcpy(h.data(), dbg_dev, blocks * 64, hipMemcpyDeviceToHost);
-            unsigned long long t0 = ~0ull;
-            for (long b = 0; b < blocks; b++) t0 = h[b * 8] < t0 ? h[b * 8] : t0;
-            double avg[5] = {0}, mx[5] = {0};
-            for (long b = 0; b < blocks; b++)
-                for (int i = 0; i < 5; i++) { double v = (double)(h[b * 8 + i] - t0) * 0.01; avg[i] += v / blocks; mx[i] = v > mx[i] ? v : mx[i]; }
-            fprintf(stderr, "dbg times us (avg/max since first start) blocks=%ld:", blocks);
-            for (int i = 0; i < 5; i++) fprintf(stderr, " [%d] %.2f/%.2f", i, avg[i], mx[i]);
-            fprintf(stderr, "\n");
-        }
-#endif
         if (p.split > 1) {
             inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq)), dim3((unsigned)inst->threads), 0, 0>>>(p);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }

@@ -65,6 +65,8 @@ lib.zk_gemm_get_path.restype = _ci
 lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
 lib.zk_timer_stop_ms.restype = ctypes.c_float
 lib.zk_gemm_guard_hits.restype = ctypes.c_long
+lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
+lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
 
 
 def _check(what):
