@@ -124,30 +124,37 @@ __device__ __noinline__ int64_t rms_apply_slow(int64_t a, int64_t w, int64_t r)
     return (int64_t)(uint64_t)(u128)qq;
 }
 
-// Fast exact path for 0 < r < 2^62 and |quotient| < 2^49: a double estimate of the quotient is within one
-// of the floor; the remainder, exact modulo 2^64, settles it.  Anything else takes the slow path.
-__device__ __forceinline__ int64_t rms_apply_one(int64_t a, int64_t w, int64_t r, double inv_r, bool fast_r)
+// Fast exact path for 0 < r < 2^62 and |quotient| < 2^49.  The quotient is estimated in double precision from
+// the operands themselves: a, w and 1/r each carry a relative error of at most 2^-53 and so does each of the two
+// products, so the estimate is off by less than 2^49 * 5 * 2^-53 < 0.32 and, rounded to nearest, lands within
+// one of the floor.  The remainder, exact modulo 2^64, settles which; anything else takes the slow path.
+// The rounding and the conversion to an integer are one addition: for |x| < 2^51 the low bits of
+// x + 1.5 * 2^52 hold round(x) as a fixed-point number.
+template <typename WT>
+__device__ __forceinline__ int64_t rms_apply_one(int64_t a, WT w, int64_t r, double inv_r, bool fast_r)
 {
     if (fast_r) {
-        uint64_t plo = (uint64_t)a * (uint64_t)w;
-        int64_t phi = __mul64hi((long long)a, (long long)w);
-        double pd = (double)phi * 18446744073709551616.0 + (double)plo;
-        double qd = floor(pd * inv_r);
-        if (fabs(qd) < 562949953421312.0) {
-            int64_t q = (int64_t)qd;
+        const double xd = (double)a * (double)w * inv_r;
+        if (fabs(xd) < 562949953421312.0) {
+            const double magic = 6755399441055744.0;
+            int64_t q = __double_as_longlong(xd + magic) - __double_as_longlong(magic);
+            const uint64_t plo = (uint64_t)a * (uint64_t)(int64_t)w;
             int64_t rem = (int64_t)(plo - (uint64_t)q * (uint64_t)r);
             if (rem < 0) { q--; rem += r; }
-            if (rem < 0) { q--; rem += r; }
-            if (rem >= r) { q++; rem -= r; }
-            if (rem >= r) { q++; rem -= r; }
+            else if (rem >= r) { q++; rem -= r; }
             if (rem >= 0 && rem < r) return q;
         }
     }
-    return rms_apply_slow(a, w, r);
+    return rms_apply_slow(a, (int64_t)w, r);
 }
 
 constexpr int kRmsThreads = 256;
+#ifndef ZK_RMS_T8K
+#define ZK_RMS_T8K 512
+#define ZK_RMS_E8K 16
+#endif
 
+template <int THREADS>
 __device__ __forceinline__ U192 block_sum_u192(U192 acc, U192 *red)
 {
     acc = wave_sum_u192(acc);
@@ -156,7 +163,7 @@ __device__ __forceinline__ U192 block_sum_u192(U192 acc, U192 *red)
     __syncthreads();
     U192 tot = red[0];
 #pragma unroll
-    for (int w = 1; w < kRmsThreads / 64; w++) u192_add(tot, red[w]);
+    for (int w = 1; w < THREADS / 64; w++) u192_add(tot, red[w]);
     return tot;
 }
 
@@ -168,12 +175,16 @@ __global__ __launch_bounds__(kRmsThreads) void rms_stat_kernel(const int64_t *__
     const int64_t *a = A + (long)blockIdx.x * N;
     U192 acc = { 0, 0, 0 };
     for (int i = threadIdx.x; i < N; i += kRmsThreads) u192_add_square(acc, a[i]);
-    U192 tot = block_sum_u192(acc, red);
+    U192 tot = block_sum_u192<kRmsThreads>(acc, red);
     if (threadIdx.x == 0) rms[blockIdx.x] = rms_finalize(tot, eps, dim);
 }
 
-// Normalisation only, rms given (the reference's rms_norm_32 / rms_norm_64 contract).
-template <typename WT>
+typedef int v4i_r __attribute__((ext_vector_type(4)));
+
+// Normalisation only, rms given (the reference's rms_norm_32 / rms_norm_64 contract).  A workgroup covers
+// 256 * kApplyEpt consecutive elements of one row; VEC: N is even and the rows are 16-byte aligned.
+constexpr int kApplyEpt = 8;
+template <typename WT, bool VEC>
 __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
                                                                 const int64_t *__restrict__ rms, int64_t *__restrict__ C,
                                                                 int N)
@@ -182,20 +193,48 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
     const int64_t r = rms[row];
     const bool fast_r = r > 0 && r < ((int64_t)1 << 62);
     const double inv_r = fast_r ? 1.0 / (double)r : 0.0;
-    int i = blockIdx.x * kRmsThreads + threadIdx.x;
-    if (i < N) C[row * N + i] = rms_apply_one(A[row * N + i], (int64_t)W[i], r, inv_r, fast_r);
+    const int base = blockIdx.x * (kRmsThreads * kApplyEpt);
+    const int64_t *a = A + row * N;
+    int64_t *c = C + row * N;
+    if (VEC) {
+        v4i_r t[kApplyEpt / 2];
+#pragma unroll
+        for (int j = 0; j < kApplyEpt / 2; j++) {
+            const int i = base + (j * kRmsThreads + threadIdx.x) * 2;
+            if (i < N) t[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
+        }
+#pragma unroll
+        for (int j = 0; j < kApplyEpt / 2; j++) {
+            const int i = base + (j * kRmsThreads + threadIdx.x) * 2;
+            if (i < N) {
+                const int64_t v0 = (int64_t)(((uint64_t)(uint32_t)t[j][1] << 32) | (uint32_t)t[j][0]);
+                const int64_t v1 = (int64_t)(((uint64_t)(uint32_t)t[j][3] << 32) | (uint32_t)t[j][2]);
+                const int64_t c0 = rms_apply_one(v0, W[i], r, inv_r, fast_r);
+                const int64_t c1 = rms_apply_one(v1, W[i + 1], r, inv_r, fast_r);
+                const v4i_r o = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
+                                  (int)(uint32_t)((uint64_t)c1 >> 32) };
+                __builtin_nontemporal_store(o, reinterpret_cast<v4i_r *>(c + i));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kApplyEpt; j++) {
+            const int i = base + j * kRmsThreads + threadIdx.x;
+            if (i < N) c[i] = rms_apply_one(a[i], W[i], r, inv_r, fast_r);
+        }
+    }
 }
 
-typedef int v4i_r __attribute__((ext_vector_type(4)));
-
-// Statistic + normalisation, one workgroup per row, the row kept in registers (N <= 256 * EPT).
+// Statistic + normalisation, one workgroup of THREADS per row, the row kept in registers (N <= THREADS * EPT).
+// Long rows get more threads rather than more elements per thread: fewer registers mean more rows in flight per
+// compute unit, which is what hides the serial stretch (reduction, division, square root) in the middle.
 // VEC: N is even and the rows are 16-byte aligned: elements are moved two at a time with streaming accesses.
-template <typename WT, int EPT, bool VEC>
-__global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
+template <typename WT, int THREADS, int EPT, bool VEC>
+__global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
                                                                 int64_t *__restrict__ rms, int64_t *__restrict__ C,
                                                                 int N, int64_t eps, int64_t dim)
 {
-    __shared__ U192 red[kRmsThreads / 64];
+    __shared__ U192 red[THREADS / 64];
     __shared__ int64_t rms_s;
     const long row = blockIdx.x;
     const int64_t *a = A + row * N;
@@ -204,7 +243,7 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     if (VEC) {
 #pragma unroll
         for (int j = 0; j < EPT / 2; j++) {
-            const int i = (j * kRmsThreads + threadIdx.x) * 2;
+            const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
                 const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
                 v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
@@ -216,11 +255,11 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     } else {
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
-            const int i = j * kRmsThreads + threadIdx.x;
+            const int i = j * THREADS + threadIdx.x;
             if (i < N) { v[j] = a[i]; u192_add_square(acc, v[j]); }
         }
     }
-    U192 tot = block_sum_u192(acc, red);
+    U192 tot = block_sum_u192<THREADS>(acc, red);
     if (threadIdx.x == 0) {
         int64_t r = rms_finalize(tot, eps, dim);
         rms_s = r;
@@ -233,10 +272,10 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     if (VEC) {
 #pragma unroll
         for (int j = 0; j < EPT / 2; j++) {
-            const int i = (j * kRmsThreads + threadIdx.x) * 2;
+            const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
-                const int64_t c0 = rms_apply_one(v[2 * j], (int64_t)W[i], r, inv_r, fast_r);
-                const int64_t c1 = rms_apply_one(v[2 * j + 1], (int64_t)W[i + 1], r, inv_r, fast_r);
+                const int64_t c0 = rms_apply_one(v[2 * j], W[i], r, inv_r, fast_r);
+                const int64_t c1 = rms_apply_one(v[2 * j + 1], W[i + 1], r, inv_r, fast_r);
                 const v4i_r t = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
                                   (int)(uint32_t)((uint64_t)c1 >> 32) };
                 __builtin_nontemporal_store(t, reinterpret_cast<v4i_r *>(C + row * N + i));
@@ -245,8 +284,8 @@ __global__ __launch_bounds__(kRmsThreads) void rms_fused_kernel(const int64_t *_
     } else {
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
-            const int i = j * kRmsThreads + threadIdx.x;
-            if (i < N) C[row * N + i] = rms_apply_one(v[j], (int64_t)W[i], r, inv_r, fast_r);
+            const int i = j * THREADS + threadIdx.x;
+            if (i < N) C[row * N + i] = rms_apply_one(v[j], W[i], r, inv_r, fast_r);
         }
     }
 }
@@ -264,8 +303,11 @@ static void launch_apply(const char *name, const int64_t *A, const WT *W, const 
 {
     if (!rms_args_ok(name, A, W, rms, C, M, N)) return;
     if (M > 65535) { set_error(kUnsupportedSize, "%s: more than 65535 rows", name); return; }
-    dim3 grid((unsigned)((N + kRmsThreads - 1) / kRmsThreads), (unsigned)M);
-    rms_apply_kernel<WT><<<grid, dim3(kRmsThreads), 0, 0>>>(A, W, rms, C, N);
+    const int per_wg = kRmsThreads * kApplyEpt;
+    dim3 grid((unsigned)((N + per_wg - 1) / per_wg), (unsigned)M);
+    const bool vec = N % 2 == 0 && (((uintptr_t)A | (uintptr_t)C) & 15) == 0;
+    if (vec) rms_apply_kernel<WT, true><<<grid, dim3(kRmsThreads), 0, 0>>>(A, W, rms, C, N);
+    else rms_apply_kernel<WT, false><<<grid, dim3(kRmsThreads), 0, 0>>>(A, W, rms, C, N);
     check_launch(name);
 }
 
@@ -281,22 +323,24 @@ static void launch_fused(const char *name, const int64_t *A, const WT *W, int64_
                          int64_t eps, int64_t dim)
 {
     if (!rms_args_ok(name, A, W, rms, C, M, N) || !stat_args_ok(name, eps, dim)) return;
-    dim3 grid((unsigned)M), block(kRmsThreads);
     const bool vec = N % 2 == 0 && (((uintptr_t)A | (uintptr_t)C) & 15) == 0;
-    if (N <= kRmsThreads * 2) {
-        if (vec) rms_fused_kernel<WT, 2, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-        else rms_fused_kernel<WT, 2, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    } else if (N <= kRmsThreads * 8) {
-        if (vec) rms_fused_kernel<WT, 8, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-        else rms_fused_kernel<WT, 8, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    } else if (N <= kRmsThreads * 32) {
-        if (vec) rms_fused_kernel<WT, 32, true><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-        else rms_fused_kernel<WT, 32, false><<<grid, block, 0, 0>>>(A, W, rms, C, N, eps, dim);
-    } else {
-        rms_stat_kernel<<<grid, block, 0, 0>>>(A, rms, N, eps, dim);
+    const dim3 grid((unsigned)M);
+#define ZK_RMS_LAUNCH(THREADS, EPT)                                                                                   \
+    do {                                                                                                              \
+        if (vec) rms_fused_kernel<WT, THREADS, EPT, true><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);   \
+        else rms_fused_kernel<WT, THREADS, EPT, false><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);      \
+    } while (0)
+    if (N <= 512) ZK_RMS_LAUNCH(256, 2);
+    else if (N <= 2048) ZK_RMS_LAUNCH(256, 8);
+    else if (N <= 4096) ZK_RMS_LAUNCH(512, 8);
+    else if (N <= 8192) ZK_RMS_LAUNCH(ZK_RMS_T8K, ZK_RMS_E8K);
+    else if (N <= 16384) ZK_RMS_LAUNCH(1024, 16);
+    else {
+        rms_stat_kernel<<<grid, dim3(kRmsThreads), 0, 0>>>(A, rms, N, eps, dim);
         if (check_launch(name)) launch_apply<WT>(name, A, W, rms, C, M, N);
         return;
     }
+#undef ZK_RMS_LAUNCH
     check_launch(name);
 }
 
