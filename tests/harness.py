@@ -109,6 +109,92 @@ class GpuBackend:
         return y
 
 
+class CheckedGpuBackend(GpuBackend):
+    """GpuBackend that checks every kernel call against the CPU oracle on the call's ACTUAL inputs: completely
+    when the call is small, on a seeded sample of output rows/columns/heads otherwise.  A chain run through it
+    is verified link by link at sizes where a whole-chain CPU run would take hours."""
+
+    def __init__(self, kernel, cpu, seed=0, full_limit=1 << 27):
+        super().__init__(kernel)
+        self.cpu = cpu
+        self.rng = np.random.default_rng(seed)
+        self.full_limit = full_limit          # multiply-adds (or elements) up to which a call is checked in full
+        self.checked = {}
+
+    def _count(self, what, n):
+        self.checked[what] = self.checked.get(what, 0) + int(n)
+
+    def _pick(self, n, k):
+        if n <= k:
+            return np.arange(n)
+        return np.unique(np.concatenate([[0, n - 1], self.rng.integers(0, n, k - 2)]))
+
+    def _dev(self, idx):
+        return self.t.from_numpy(np.asarray(idx, dtype=np.int64)).cuda()
+
+    def linear(self, x, w, shift):
+        C, R = super().linear(x, w, shift)
+        M, K, N = x.shape[1], x.shape[2], w.shape[0]
+        rows = np.arange(M) if M * N * K <= self.full_limit else self._pick(M, 3)
+        cols = np.arange(N) if M * N * K <= self.full_limit else self._pick(N, 48)
+        xr, wc = x[:, self._dev(rows)], w[self._dev(cols)]
+        Ce, Re = self.cpu.linear(xr.cpu().numpy(), wc.cpu().numpy(), shift)
+        sub = lambda t: t[:, self._dev(rows)][:, :, self._dev(cols)].cpu().numpy()
+        assert np.array_equal(sub(C), Ce), "linear: quotient differs from the oracle"
+        assert np.array_equal(sub(R), Re), "linear: remainder differs from the oracle"
+        self._count("linear", rows.size * cols.size)
+        return C, R
+
+    def _rowwise(self, what, gpu_fn, cpu_fn, x):
+        out = gpu_fn(x)
+        flat_in, flat_out = x.reshape(-1, x.shape[-1]), out.reshape(-1, x.shape[-1])
+        rows = np.arange(flat_in.shape[0]) if x.numel() <= self.full_limit else self._pick(flat_in.shape[0], 4096)
+        got = flat_out[self._dev(rows)].cpu().numpy()
+        want = cpu_fn(np.ascontiguousarray(flat_in[self._dev(rows)].cpu().numpy()))
+        assert np.array_equal(got, want), what + " differs from the oracle"
+        self._count(what, got.size)
+        return out
+
+    def silu(self, x):
+        return self._rowwise("silu", super().silu, self.cpu.silu, x)
+
+    def sigmoid(self, x):
+        return self._rowwise("sigmoid", super().sigmoid, self.cpu.sigmoid, x)
+
+    def softmax(self, x):
+        cpu_fn = lambda rows: self.cpu.softmax(rows[None, None])[0, 0]
+        return self._rowwise("softmax", super().softmax, cpu_fn, x)
+
+    def rmsnorm(self, x2d, w, dim):
+        out = super().rmsnorm(x2d, w, dim)
+        want = self.cpu.rmsnorm(x2d.cpu().numpy(), w.cpu().numpy(), dim)
+        assert np.array_equal(out.cpu().numpy(), want), "rmsnorm differs from the oracle"
+        self._count("rmsnorm", want.size)
+        return out
+
+    def rope(self, x, table):
+        out = super().rope(x, table)
+        want = self.cpu.rope(np.ascontiguousarray(x.cpu().numpy()), np.ascontiguousarray(table.cpu().numpy()))
+        assert np.array_equal(out.cpu().numpy(), want), "rope differs from the oracle"
+        self._count("rope", want.size)
+        return out
+
+    def einsum(self, name, a, b, shift):
+        out = super().einsum(name, a, b, shift)
+        S, H = a.shape[1], a.shape[2]
+        macs = out.numel() * a.shape[3]
+        ss = np.arange(S) if macs <= self.full_limit else self._pick(S, 3)
+        hs = np.arange(H) if macs <= self.full_limit else self._pick(H, 4)
+        asub = a[:, self._dev(ss)][:, :, self._dev(hs)].contiguous().cpu().numpy()
+        per_head = name in ("einsum_bshd_hdc_bshc", "einsum_bshc_hdc_bshd")          # b is [H, D, C]
+        bsub = (b[self._dev(hs)] if per_head else b).contiguous().cpu().numpy()
+        want = self.cpu.einsum(name, asub, bsub, shift)
+        got = out[:, self._dev(ss)][:, :, self._dev(hs)].cpu().numpy()
+        assert np.array_equal(got, want), name + " differs from the oracle"
+        self._count(name, got.size)
+        return out
+
+
 def expert_ffn(be, x, w1, w2, w3, c13, c2):
     """gate/up GEMMs, SiLU gate, down GEMM: MLP_int.forward / Expert_int.forward
     (inference/model.py:1018-1049, 1247-1281).  x [1,M,dim] Q23 activations."""
@@ -138,15 +224,16 @@ def attention_scores_softmax_pv(be, q_nope, q_pe, kv_cache, pe_cache, causal=Tru
 def mla(be, x, P, freqs, cfg):
     """MLA.forward in absorb mode at start_pos = 0 (inference/model.py:747-957).  x [1,S,dim]."""
     S, H = x.shape[1], cfg["heads"]
-    q_down, _ = be.linear(x, P["wq_a"], 30)
+    cq, ckv = cfg.get("c_q", 30), cfg.get("c_kv", 29)           # the model's scales (model.py:772-833); tests may pick others
+    q_down, _ = be.linear(x, P["wq_a"], cq)
     q_normed = be.rmsnorm(q_down[0], P["q_norm"], cfg["q_lora"])[None]
-    q_nope, _ = be.linear(q_normed, P["wq_b1"], 30)
-    q_pe, _ = be.linear(q_normed, P["wq_b2"], 30)
+    q_nope, _ = be.linear(q_normed, P["wq_b1"], cq)
+    q_pe, _ = be.linear(q_normed, P["wq_b2"], cq)
     q_nope = q_nope.reshape(1, S, H, cfg["nope"])
     q_pe = q_pe.reshape(1, S, H, cfg["rope"] // 2, 2)
     q_pe = be.rope(q_pe, freqs).reshape(1, S, H, cfg["rope"])
-    kv, _ = be.linear(x, P["wkv_a1"], 29)
-    k_pe, _ = be.linear(x, P["wkv_a2"], 29)
+    kv, _ = be.linear(x, P["wkv_a1"], ckv)
+    k_pe, _ = be.linear(x, P["wkv_a2"], ckv)
     k_pe = be.rope(k_pe.reshape(1, S, 1, cfg["rope"] // 2, 2), freqs).reshape(1, S, cfg["rope"])
     q_abs = be.einsum("einsum_bshd_hdc_bshc", q_nope, P["wkv_b_1"], cfg["wkv_b_1_scale"])
     kv_normed = be.rmsnorm(kv[0], P["kv_norm"], cfg["kv_lora"])[None]

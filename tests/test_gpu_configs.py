@@ -110,3 +110,60 @@ def test_config5_decoder_layer_reduced(backends):
     assert np.array_equal(yg.cpu().numpy(), yc)
     assert len(np.unique(idx_c)) > cfg["topk"], "routing should spread over several experts"
     kernel.lib.zk_gemm_set_path(0)
+
+
+def test_config5_decoder_layer_full_size(backends):
+    """Config 5 at its real shape: one DeepSeek-V3 MoE decoder layer on 256 tokens, dim 7168, q_lora 1536, kv_lora
+    512, 128 heads (nope 128 / rope 64 / v 128), 256 routed experts of width 2048 (top-8 in 4 of 8 groups) plus
+    the shared expert, every weight resident on the GPU (90.2 GB of int64 expert weights in the config-1 value
+    range).  A CPU run of the whole layer is out of reach, so the layer runs through a back end that checks
+    EVERY kernel call against the oracle on that call's actual inputs (small calls completely, large ones on a
+    seeded sample of rows/columns/heads), which verifies the chain link by link.  The shifts are the harness's
+    choice for these value ranges (they keep every stage between 2^17 and 2^26 in magnitude): linear 18/22,
+    wkv_b 20/16, wo 22, gate 17, experts 17/20."""
+    gpu, cpu, kernel = backends
+    free, total = torch.cuda.mem_get_info()
+    if free < 110 * (1 << 30):
+        pytest.skip("needs 110 GB of free device memory, %d GB free" % (free >> 30))
+    cfg = dict(dim=7168, q_lora=1536, kv_lora=512, heads=128, nope=128, rope=64, v=128, experts=256, topk=8, groups=8,
+               topk_groups=4, inter=2048, c_q=18, c_kv=22, wkv_b_1_scale=20, wkv_b_2_scale=16, wo_scale=22,
+               gate_scale=17, c13=17, c2=20)
+    S = 256
+    gd = torch.Generator(device="cuda").manual_seed(5001)
+    w64 = lambda *shape: torch.randint(-(1 << 16), 1 << 16, shape, generator=gd, dtype=torch.int64, device="cuda")
+    w32 = lambda *shape: torch.randint(-(1 << 16), 1 << 16, shape, generator=gd, dtype=torch.int32, device="cuda")
+    norm = lambda n, lo, hi: torch.randint(lo, hi, (n,), generator=gd, dtype=torch.int32, device="cuda")
+    E, dim, inter, heads = cfg["experts"], cfg["dim"], cfg["inter"], cfg["heads"]
+    P = {
+        "attn_norm": norm(dim, 1 << 18, 1 << 20), "ffn_norm": norm(dim, 1 << 18, 1 << 20),
+        "q_norm": norm(cfg["q_lora"], 1 << 18, 1 << 20), "kv_norm": norm(cfg["kv_lora"], 1 << 20, 1 << 22),
+        "wq_a": w64(cfg["q_lora"], dim), "wq_b1": w64(heads * cfg["nope"], cfg["q_lora"]),
+        "wq_b2": w64(heads * cfg["rope"], cfg["q_lora"]), "wkv_a1": w64(cfg["kv_lora"], dim), "wkv_a2": w64(cfg["rope"], dim),
+        "wkv_b_1": w32(heads, cfg["nope"], cfg["kv_lora"]), "wkv_b_2": w32(heads, cfg["v"], cfg["kv_lora"]),
+        "wo": w64(dim, heads * cfg["v"]), "gate": w64(E, dim),
+        "w1": [w64(inter, dim) for _ in range(E)], "w3": [w64(inter, dim) for _ in range(E)],
+        "w2": [w64(dim, inter) for _ in range(E)],
+        "sw1": w64(inter, dim), "sw3": w64(inter, dim), "sw2": w64(dim, inter),
+    }
+    expert_bytes = sum(t.numel() * 8 for k in ("w1", "w2", "w3") for t in P[k])
+    assert expert_bytes == 256 * 3 * 2048 * 7168 * 8                      # 90.2 GB resident
+    gh = torch.Generator(device="cpu").manual_seed(5002)
+    P["gate_bias_host"] = _ri(gh, -(1 << 18), 1 << 18, (E,)).numpy()
+    ang = torch.rand((1, S, 1, cfg["rope"] // 2), generator=gh, dtype=torch.float64) * 6.283185307179586
+    freqs = torch.stack([torch.round(torch.cos(ang) * 2 ** 42), torch.round(torch.sin(ang) * 2 ** 42)], -1).to(torch.int64).cuda()
+    x = _ri(gh, -(1 << 20), 1 << 20, (1, S, dim)).cuda()
+
+    checked = H.CheckedGpuBackend(kernel, cpu, seed=5003, full_limit=1 << 24)
+    y, idx = H.decoder_layer(checked, x, P, freqs, cfg)
+    torch.cuda.synchronize()
+    kernel._check("config 5")
+    assert y.shape == (1, S, dim)
+    assert idx.shape == (S, cfg["topk"]) and len(np.unique(idx)) > 200, "routing should reach most of the 256 experts"
+    c = checked.checked
+    assert c["linear"] > 3 * 48 * (6 + 3 * 200) and c["softmax"] >= 4096 * S and c["rmsnorm"] == S * (2 * dim + 1536 + 512)
+    for name in ("einsum_bshd_hdc_bshc", "einsum_bshc_btc_bsht", "einsum_bsht_btc_bshc", "einsum_bshc_hdc_bshd", "silu", "sigmoid", "rope"):
+        assert c.get(name, 0) > 0, name
+    # the layer's output is alive: neither stuck at the residual nor saturated
+    d = (y - x).abs()
+    assert int(d.max()) > 0 and int(y.abs().max()) < 1 << 62
+    kernel.lib.zk_gemm_set_path(0)

@@ -79,6 +79,21 @@ def test_gemm_ragged_shapes(K, oracle, path, shape):
     _gemm_case(K, oracle, path, A, W, 1, 1, 13)
 
 
+@pytest.mark.parametrize("bits", [(20, 16), (37, 31), (45, 20)])
+@pytest.mark.parametrize("shape", [(1, 8, 512, 2048), (2, 20, 300, 1100), (1, 32, 96, 1024), (1, 3, 2048, 7168),
+                                   (1, 100, 2048, 520), (1, 40, 4096, 200)])
+def test_gemm_few_rows_many_columns(K, oracle, shape, bits):
+    """expert-FFN-like shapes: a handful of tokens against a wide weight matrix (32-row tiles, digit planes of A,
+    K split over many workgroups), and mid-sized launches that are split along K as well"""
+    Bd, M, Kd, N = shape
+    rng = np.random.default_rng(sum(shape) + bits[0])
+    A = rand_i64(rng, (Bd, M, Kd), bits[0])
+    W = rand_i64(rng, (N, Kd), bits[1])
+    for c in (0, 23):
+        _gemm_case(K, oracle, 2, A, W, 1, 1, c)
+    K.lib.zk_gemm_set_path(0)
+
+
 @pytest.mark.parametrize("path", PATHS)
 def test_gemm_operand_divisors(K, oracle, path):
     """head projection divides the weights by 256 (inference/model.py:1519); division truncates toward zero"""

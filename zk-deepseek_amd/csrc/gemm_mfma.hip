@@ -286,8 +286,10 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
     // plane step layout: [g][sub][ks32][digit][1 KB]; a step of KK depths is contiguous per sub
     unsigned char *dst = planes + (((long)g * msub + (row >> 5)) * ksteps32 + ks * KK + (j >> 2)) * (NA * 1024) +
                          ((row & 31) + 32 * ((j & 3) >> 1)) * 16 + (j & 1) * 8;
+    if (row < msub * 32) {                  // a workgroup may reach past the last 32-row group (skinny tiles)
 #pragma unroll
-    for (int i = 0; i < NA; i++) *reinterpret_cast<uint2 *>(dst + i * 1024) = dg[i];
+        for (int i = 0; i < NA; i++) *reinterpret_cast<uint2 *>(dst + i * 1024) = dg[i];
+    }
     r = mm_wave(r);
     if ((tid & 63) == 0) red[tid >> 6] = r;
     __syncthreads();
@@ -1067,7 +1069,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             if (!grow(g_cache.planes, g_cache.planes_bytes, need, "digit-plane buffer")) return false;
             p.a_planes = g_cache.planes; p.a_msub = msub; p.a_ksteps = ksteps;
             const int rows_per_wg = 256 / (4 * inst->kk);
-            const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)(msub * 32 / rows_per_wg), (unsigned)d.G);
+            const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)((msub * 32 + rows_per_wg - 1) / rows_per_wg), (unsigned)d.G);
             plane_wgs = (long)pgrid.x * pgrid.y * pgrid.z;
             if (!grow(g_cache.mm, g_cache.mm_count, (size_t)plane_wgs * 2, "range scratch")) return false;
             inst->planes[d.b32 ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
@@ -1082,7 +1084,14 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             lds_raised.insert((const void *)fn);
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
-        if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: MFMA kernel launch failed"); return false; }
+        {
+            const hipError_t err = hipGetLastError();
+            if (err != hipSuccess) {
+                set_error(kLaunchFailure, "gemm: MFMA kernel launch failed (%s; digits %d,%d, %ld workgroups of %d threads, %zu bytes of LDS)",
+                          hipGetErrorString(err), inst->na, inst->nb, blocks, inst->threads, lds);
+                return false;
+            }
+        }
         if (p.split > 1) {
             inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq)), dim3((unsigned)inst->threads), 0, 0>>>(p);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
