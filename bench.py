@@ -285,6 +285,51 @@ def cpu_leg(A_h, W_h, c):
     if cores > 8:
         dt8, _ = run(max(64, ncols // 2), 8)
         res["value_8_threads"] = 512 * 7168 * max(64, ncols // 2) / dt8 / 1e9
+
+    # config 1 on the same CPU path (Y[16,576] = X[16,7168] @ W[576,7168]^T), all cores
+    torch.set_num_threads(cores)
+    g1 = torch.Generator(device="cpu").manual_seed(1000)
+    X1 = randint(g1, -(1 << 20), 1 << 20, (16, 7168))
+    W1t = randint(g1, -(1 << 16), 1 << 16, (576, 7168)).T.contiguous()
+    torch.matmul(X1, W1t)
+    t0 = time.perf_counter()
+    for _ in range(20):
+        y1 = torch.matmul(X1, W1t) >> c
+    dt1 = (time.perf_counter() - t0) / 20
+    res["config1_gmacs"] = 16 * 7168 * 576 / dt1 / 1e9
+
+    # The reference has no CPU implementation of its fixed-point kernels; what is timed here is this build's scalar
+    # C restatement of them (OpenMP over rows), labelled as such: "oracle, not reference".
+    try:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import numpy as np
+        import oracle
+        oracle.set_threads(cores)
+        rng = np.random.default_rng(7)
+        others = {}
+
+        def leg(name, fn, nelem, what):
+            fn()
+            reps, t0 = 0, time.perf_counter()
+            while reps < 3 or time.perf_counter() - t0 < 2.0:
+                fn()
+                reps += 1
+            dt = (time.perf_counter() - t0) / reps
+            others[name] = {"value": nelem * 16.0 / dt / 1e9, "unit": "GB/s at 16 B/element", "cores": cores,
+                            "kind": "port (oracle, not reference)",
+                            "sample": "%s, %d passes of %.1f ms" % (what, reps, dt * 1e3)}
+
+        xs = rng.integers(-(6 << 19), 6 << 19, size=(1, 64, 128, 1024), dtype=np.int64)
+        leg("softmax_q19", lambda: oracle.softmax_q19(xs), xs.size, "rows of config 3: [1,64,128,1024]")
+        xa = rng.integers(-(16 << 23), 16 << 23, size=(1, 512, 18432), dtype=np.int64)
+        leg("silu_q23", lambda: oracle.silu_q23(xa), xa.size, "[1,512,18432]")
+        xr = rng.integers(-(1 << 37), 1 << 37, size=(2048, 7168), dtype=np.int64)
+        wr = rng.integers(1 << 18, 1 << 20, size=(7168,), dtype=np.int64).astype(np.int32)
+        leg("rmsnorm", lambda: oracle.RMS_Norm_int64(xr, wr, 1, 7168), xr.size, "[2048,7168], int32 weights")
+        oracle.set_threads(1)
+        res["fixed_point_kernels"] = others
+    except Exception as e:                                  # the CPU legs are a reported baseline, never a reason to fail
+        res["fixed_point_kernels"] = {"error": repr(e)}
     return res
 
 
