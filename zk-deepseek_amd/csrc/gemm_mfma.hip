@@ -866,6 +866,7 @@ constexpr int kPendingSlots = 16;
 struct RangeCache {
     std::mutex mu;
     std::map<OperandKey, int> limbs;         // operand -> digits its values needed when last seen
+    std::map<OperandKey, int> partner_a;     // B operand -> digits of the A operand it was last multiplied with
     unsigned long long *dev = nullptr;       // [minA, maxA, minB, maxB, verdict]
     unsigned char *planes = nullptr;         // digit planes of A, grown on demand, kept for the process lifetime
     size_t planes_bytes = 0;
@@ -889,6 +890,13 @@ struct RangeCache {
     {
         if (limbs.size() > 4096) limbs.clear();
         limbs[k] = n;
+    }
+    void store_pair(const OperandKey &ka, int na, const OperandKey &kb, int nb)
+    {
+        store(ka, na);
+        store(kb, nb);
+        if (partner_a.size() > 4096) partner_a.clear();
+        partner_a[kb] = na;
     }
 };
 
@@ -924,8 +932,8 @@ static void drain_pending()
         const hipError_t st = hipEventQuery(s.ev);
         if (st != hipSuccess) { (void)hipGetLastError(); if (st == hipErrorNotReady) continue; }
         if (st == hipSuccess) {
-            g_cache.store(s.key_a, limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip)));
-            g_cache.store(s.key_b, limbs_needed((int64_t)(s.host[2] ^ kSignFlip), (int64_t)(s.host[3] ^ kSignFlip)));
+            g_cache.store_pair(s.key_a, limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip)),
+                               s.key_b, limbs_needed((int64_t)(s.host[2] ^ kSignFlip), (int64_t)(s.host[3] ^ kSignFlip)));
             if (s.host[4]) g_cache.guard_hits++;
         }
         s.busy = false;
@@ -981,6 +989,12 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
 
     const OperandKey key_a(d.A, (long)d.G * d.M, d.K, 8), key_b(d.B, d.N, d.K, d.b32 ? 4 : 8);
     int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
+    // Activations gathered into a fresh buffer for a known weight matrix (the experts of a MoE layer): guess the
+    // digits the last activations multiplied with that matrix needed.  A wrong guess costs one guarded recomputation.
+    if (!na && nb) {
+        auto it = g_cache.partner_a.find(key_b);
+        if (it != g_cache.partner_a.end()) na = it->second;
+    }
     // Operands seen before: speculate, do not wait.  Otherwise sample them and check the verdict before returning.
     PendingRange *slot = nullptr;
     if (na && nb && g_cache.pinned && getenv("ZK_GEMM_SYNC") == nullptr) {
@@ -1013,8 +1027,9 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (per_batch > 0x7FFFFFFFL) return false;
         const long total = per_batch * d.G;
         if (total > 0x7FFFFFFFL / 8) return false;
-        // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass
-        const bool use_planes = !kmajor && p.tiles_n >= 4;
+        // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass (never for the
+        // 32-row tiles: splitting a handful of rows on the fly is cheaper than another kernel in front)
+        const bool use_planes = !kmajor && p.tiles_n >= 4 && !inst->skinny;
         const int variant = kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
@@ -1116,8 +1131,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
-        g_cache.store(key_a, need_a);
-        g_cache.store(key_b, need_b);
+        g_cache.store_pair(key_a, need_a, key_b, need_b);
         if (need_a <= inst->na && need_b <= inst->nb) return true;
         na = need_a;
         nb = need_b;
