@@ -211,6 +211,25 @@ def main():
                 Ar.numel(), extra_bytes=4.0 * 7168 + 8.0 * Mr, steps=20)
             del Ar, Cr
 
+        # RoPE and the float -> fixed converters (weight-loading path), by their own algorithmic bytes per element
+        gq = torch.Generator(device="cpu").manual_seed(700)
+        q_pe = randint(gq, -(1 << 30), 1 << 30, (1, 4096, 128, 32, 2)).cuda()
+        tab = randint(gq, -(1 << 42), 1 << 42, (1, 4096, 1, 32, 2)).cuda()
+        out = torch.empty_like(q_pe)
+        hbm("rope_1x4096x128x64", lambda: K.lib.complex_int64_mul(q_pe.data_ptr(), tab.data_ptr(), out.data_ptr(), 1, 4096, 128, 32),
+            q_pe.numel(), steps=20)
+        del q_pe, out
+        wb = torch.randn((18432, 7168), generator=gq, dtype=torch.float32)
+        w16 = wb.to(torch.bfloat16).cuda()
+        o32 = torch.empty((18432, 7168), dtype=torch.int32, device="cuda")
+        hbm("bf16_to_int32_18432x7168", lambda: K.lib.bf16_to_int32_2d(w16.data_ptr(), o32.data_ptr(), 18432, 7168, 20),
+            w16.numel(), bytes_per_elem=6.0, steps=20)
+        w32 = wb.cuda()
+        o64 = torch.empty((18432, 7168), dtype=torch.int64, device="cuda")
+        hbm("float32_to_int64_18432x7168", lambda: K.lib.float32_to_int64_2d(w32.data_ptr(), o64.data_ptr(), 18432, 7168, 5),
+            w32.numel(), bytes_per_elem=12.0, steps=20)
+        del wb, w16, o32, w32, o64
+
     if "calib" in legs:
         # plain copy of known size (1 GiB in, 1 GiB out): what FETCH_SIZE / WRITE_SIZE read for it is the
         # scale factor applied to the same counters of the GEMM kernel (see profiles/)

@@ -515,4 +515,18 @@ def test_converters(K, oracle):
     o32 = torch.empty((37, 129), dtype=torch.int32, device="cuda")
     K.lib.wkv_b_bf16_to_int32(src16.data_ptr(), o32.data_ptr(), 37, 129)
     assert np.array_equal(host(o32), oracle.wkv_b_bf16_to_int32(bits16))
+    # pointers that are not 16-byte aligned take the scalar kernels; a length that is no multiple of the vector
+    # width ends in a scalar tail
+    big16 = torch.from_numpy(np.concatenate([bits16.ravel(), bits16.ravel()[:7]]).view(np.int16)).cuda()
+    out = torch.empty((big16.numel(),), dtype=torch.int32, device="cuda")
+    n = big16.numel() - 1
+    K.lib.bf16_to_int32_2d(big16.data_ptr() + 2, out.data_ptr() + 4, 1, n, 12)
+    want = oracle.bf16_to_int32_2d(big16.cpu().numpy().view(np.uint16)[1:].reshape(1, n), 12)
+    assert np.array_equal(host(out)[1:], want.ravel())
+    big32 = torch.from_numpy(np.concatenate([bits32.ravel(), bits32.ravel()[:3]]).view(np.int32)).cuda()
+    out64 = torch.empty((big32.numel(),), dtype=torch.int64, device="cuda")
+    n = big32.numel() - 1
+    K.lib.float32_to_int64_2d(big32.data_ptr() + 4, out64.data_ptr() + 8, 1, n, 12)
+    want = oracle.float32_to_int64_2d(big32.cpu().numpy().view(np.uint32)[1:].reshape(1, n), 12)
+    assert np.array_equal(host(out64)[1:], want.ravel())
     K._check("converters")

@@ -276,42 +276,101 @@ __global__ __launch_bounds__(256) void rope_kernel(const i64x2 *__restrict__ A, 
 // -------------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t scale_mantissa_u32(uint32_t r2, int ex2)
 {
-    if (ex2 >= 0) return ex2 >= 32 ? 0u : r2 * (1u << ex2);
-    return -ex2 >= 31 ? 0u : r2 / (1u << -ex2);
+    // multiplying or dividing the (positive) mantissa by 1u << n is a shift
+    if (ex2 >= 0) return ex2 >= 32 ? 0u : r2 << ex2;
+    return -ex2 >= 31 ? 0u : r2 >> -ex2;
 }
 
+__device__ __forceinline__ int32_t bf16_one(uint32_t v0, int rescale, int wkv_b)
+{
+    const int ex0 = (int)((v0 >> 7) & 0xFF) - 127;
+    const int r0 = (int)(v0 & 0x7F);
+    if (ex0 == -127 && r0 == 0) return 0;
+    if (wkv_b && ex0 >= -1) return 0x7FFFFFFF;                      // saturate |x| >= 0.5 (:151-154)
+    uint32_t v = scale_mantissa_u32((uint32_t)(r0 + 128), ex0 + rescale);
+    if (v0 & 0x8000) v = 0u - v;
+    return (int32_t)v;
+}
+
+__device__ __forceinline__ int64_t f32_one(uint32_t v0, int rescale)
+{
+    const int ex0 = (int)((v0 >> 23) & 0xFF) - 127;
+    const int r0 = (int)(v0 & 0x7FFFFF);
+    if (ex0 == -127 && r0 == 0) return 0;
+    const int ex2 = ex0 + rescale;
+    const int64_t r2 = (int64_t)r0 + 8388608;
+    int64_t v;
+    // the reference multiplies by a 32-bit `1 << ex2` (:202): the factor wraps to INT_MIN at 31 and is 0 beyond
+    // (shifts instead of the multiply and the divide: the mantissa is positive; at 31 the factor is -2^31)
+    if (ex2 >= 0) v = ex2 >= 32 ? 0 : (ex2 == 31 ? (int64_t)(0 - ((uint64_t)r2 << 31)) : (int64_t)((uint64_t)r2 << ex2));
+    else v = -ex2 >= 31 ? 0 : r2 >> -ex2;
+    if (v0 & 0x80000000u) v = (int64_t)(0 - (uint64_t)v);
+    return v;
+}
+
+typedef int v4i_e __attribute__((ext_vector_type(4)));
+
+typedef int v2i_e __attribute__((ext_vector_type(2)));
+
+// Four rounds per thread; in a round adjacent lanes handle adjacent groups of four bf16 values (8-byte load, 16-byte
+// store), so loads and stores of a wavefront are both contiguous.  VEC: input 8-byte and output 16-byte aligned.
+template <bool VEC>
 __global__ __launch_bounds__(256) void bf16_to_int32_kernel(const uint16_t *__restrict__ in, int32_t *__restrict__ out,
                                                             long n, int rescale, int wkv_b)
 {
-    long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    int v0 = in[idx];
-    int ex0 = ((v0 >> 7) & 0xFF) - 127;
-    int r0 = v0 & 0x7F;
-    if (ex0 == -127 && r0 == 0) { out[idx] = 0; return; }
-    if (wkv_b && ex0 >= -1) { out[idx] = 0x7FFFFFFF; return; }       // saturate |x| >= 0.5 (:151-154)
-    uint32_t v = scale_mantissa_u32((uint32_t)(r0 + 128), ex0 + rescale);
-    if (v0 & 0x8000) v = 0u - v;
-    out[idx] = (int32_t)v;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const long base = (((long)blockIdx.x * 4 + j) * 256 + threadIdx.x) * 4;
+        if (base >= n) return;
+        if (VEC && base + 4 <= n) {
+            const v2i_e t = __builtin_nontemporal_load(reinterpret_cast<const v2i_e *>(in + base));
+            v4i_e o;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint32_t w = (uint32_t)t[h];
+                o[2 * h] = bf16_one(w & 0xFFFF, rescale, wkv_b);
+                o[2 * h + 1] = bf16_one(w >> 16, rescale, wkv_b);
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<v4i_e *>(out + base));
+        } else {
+            for (long i = base; i < base + 4 && i < n; i++) out[i] = bf16_one(in[i], rescale, wkv_b);
+        }
+    }
 }
 
+// Same shape for fp32 -> int64: two values per lane and round (8-byte load, 16-byte store).
+template <bool VEC>
 __global__ __launch_bounds__(256) void f32_to_int64_kernel(const uint32_t *__restrict__ in, int64_t *__restrict__ out,
                                                            long n, int rescale)
 {
-    long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    uint32_t v0 = in[idx];
-    int ex0 = (int)((v0 >> 23) & 0xFF) - 127;
-    int r0 = (int)(v0 & 0x7FFFFF);
-    if (ex0 == -127 && r0 == 0) { out[idx] = 0; return; }
-    int ex2 = ex0 + rescale;
-    int64_t r2 = (int64_t)r0 + 8388608;
-    int64_t v;
-    // the reference multiplies by a 32-bit `1 << ex2` (:202): the factor wraps to INT_MIN at 31 and is 0 beyond
-    if (ex2 >= 0) v = ex2 >= 32 ? 0 : (int64_t)((uint64_t)r2 * (uint64_t)(int64_t)(int32_t)(1u << ex2));
-    else v = -ex2 >= 31 ? 0 : r2 / (int64_t)(1u << -ex2);
-    if (v0 & 0x80000000u) v = (int64_t)(0 - (uint64_t)v);
-    out[idx] = v;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const long base = (((long)blockIdx.x * 4 + j) * 256 + threadIdx.x) * 2;
+        if (base >= n) return;
+        if (VEC && base + 2 <= n) {
+            const v2i_e t = __builtin_nontemporal_load(reinterpret_cast<const v2i_e *>(in + base));
+            const int64_t a = f32_one((uint32_t)t[0], rescale), b = f32_one((uint32_t)t[1], rescale);
+            const v4i_e o = { (int)(uint32_t)a, (int)(uint32_t)((uint64_t)a >> 32), (int)(uint32_t)b, (int)(uint32_t)((uint64_t)b >> 32) };
+            __builtin_nontemporal_store(o, reinterpret_cast<v4i_e *>(out + base));
+        } else {
+            for (long i = base; i < base + 2 && i < n; i++) out[i] = f32_one(in[i], rescale);
+        }
+    }
+}
+
+static void launch_bf16(const char *name, const uint16_t *input, int32_t *output, int rows, int cols, int rescale, int wkv_b)
+{
+    const long n = (long)rows * cols;
+    if (rows < 0 || cols < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
+    if (n == 0) return;
+    if (!input || !output) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    const long blocks = (n + 4095) / 4096;
+    if (blocks > 0x7FFFFFFFL) { set_error(kUnsupportedSize, "%s: too many elements", name); return; }
+    if (((uintptr_t)input & 7) == 0 && ((uintptr_t)output & 15) == 0)
+        bf16_to_int32_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, 0>>>(input, output, n, rescale, wkv_b);
+    else
+        bf16_to_int32_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, 0>>>(input, output, n, rescale, wkv_b);
+    check_launch(name);
 }
 
 }  // namespace zk
@@ -358,29 +417,28 @@ void complex_int64_mul(const int64_t *A, const int64_t *B, int64_t *C, int batch
 
 void bf16_to_int32_2d(const uint16_t *input, int32_t *output, int rows, int cols, int rescale)
 {
-    long n = (long)rows * cols;
-    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "bf16_to_int32_2d: negative dimension"); return; }
-    if (n == 0) return;
-    zk::bf16_to_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, rescale, 0);
-    zk::check_launch("bf16_to_int32_2d");
+    zk::launch_bf16("bf16_to_int32_2d", input, output, rows, cols, rescale, 0);
 }
 
 void wkv_b_bf16_to_int32(const uint16_t *input, int32_t *output, int rows, int cols)
 {
-    long n = (long)rows * cols;
-    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "wkv_b_bf16_to_int32: negative dimension"); return; }
-    if (n == 0) return;
-    zk::bf16_to_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, 25, 1);
-    zk::check_launch("wkv_b_bf16_to_int32");
+    zk::launch_bf16("wkv_b_bf16_to_int32", input, output, rows, cols, 25, 1);
 }
 
 void float32_to_int64_2d(const uint32_t *input, int64_t *output, int rows, int cols, int rescale)
 {
-    long n = (long)rows * cols;
-    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "float32_to_int64_2d: negative dimension"); return; }
+    const char *name = "float32_to_int64_2d";
+    const long n = (long)rows * cols;
+    if (rows < 0 || cols < 0) { zk::set_error(zk::kBadArgument, "%s: negative dimension", name); return; }
     if (n == 0) return;
-    zk::f32_to_int64_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(input, output, n, rescale);
-    zk::check_launch("float32_to_int64_2d");
+    if (!input || !output) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    const long blocks = (n + 2047) / 2048;
+    if (blocks > 0x7FFFFFFFL) { zk::set_error(zk::kUnsupportedSize, "%s: too many elements", name); return; }
+    if (((uintptr_t)input & 7) == 0 && ((uintptr_t)output & 15) == 0)
+        zk::f32_to_int64_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, 0>>>(input, output, n, rescale);
+    else
+        zk::f32_to_int64_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, 0>>>(input, output, n, rescale);
+    zk::check_launch(name);
 }
 
 }  // extern "C"
