@@ -211,6 +211,38 @@ def main():
                 Ar.numel(), extra_bytes=4.0 * 7168 + 8.0 * Mr, steps=20)
             del Ar, Cr
 
+        # the two fusions against the chains they replace (the reference's tensor ops around the kernel, on torch)
+        g7 = torch.Generator(device="cpu").manual_seed(3300)
+        s1 = randint(g7, -(6 << 20), 6 << 20, (1, 1024, 128, 1024)).cuda()
+        s2 = randint(g7, -(6 << 20), 6 << 20, (1, 1024, 128, 1024)).cuda()
+        msk = torch.full((1024, 1024), -(64 << 36), dtype=torch.int64).triu_(1).cuda()
+        sc = torch.empty_like(s1)
+        pr = torch.empty_like(s1)
+        hbm("softmax_q19_scores_fused_1x1024x128x1024_32B_per_element",
+            lambda: K.softmax_q19_scores(s1, s2, msk, pr, sc), s1.numel(), bytes_per_elem=32.0, steps=10)
+
+        def chain():
+            x = (s1 + s2) * 94 // 695
+            x += msk.unsqueeze(1)
+            K.lib.softmax_q19(x.data_ptr(), pr.data_ptr(), K.EXP2_FRAC_LUT_Q19.data_ptr(), 1, 1024, 128, 1024)
+
+        ms_chain = timed(K, chain, 5, 2)
+        extra["softmax_q19_scores_fused_1x1024x128x1024_32B_per_element"]["unfused_chain_ms"] = ms_chain
+        del s1, s2, sc, pr
+        g8 = torch.Generator(device="cpu").manual_seed(2400)
+        r1 = randint(g8, -(16 << 23), 16 << 23, (1, 8192, 18432)).cuda()
+        r2 = randint(g8, -(16 << 23), 16 << 23, (1, 8192, 18432)).cuda()
+        hh = torch.empty_like(r1)
+        hbm("silu_mul_q23_fused_1x8192x18432_24B_per_element", lambda: K.silu_mul_q23(r1, r2, hh), r1.numel(),
+            bytes_per_elem=24.0, steps=10)
+
+        def chain2():
+            K.lib.silu_q23(r1.data_ptr(), hh.data_ptr(), K.EXP2_FRAC_LUT_Q23.data_ptr(), 1, 8192, 18432)
+            torch.bitwise_right_shift(hh * r2, 23, out=hh)
+
+        extra["silu_mul_q23_fused_1x8192x18432_24B_per_element"]["unfused_chain_ms"] = timed(K, chain2, 5, 2)
+        del r1, r2, hh
+
         # RoPE and the float -> fixed converters (weight-loading path), by their own algorithmic bytes per element
         gq = torch.Generator(device="cpu").manual_seed(700)
         q_pe = randint(gq, -(1 << 30), 1 << 30, (1, 4096, 128, 32, 2)).cuda()

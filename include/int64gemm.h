@@ -114,6 +114,20 @@ void rms_norm_fused_64(const int64_t *A, const int64_t *W, int64_t *rms, int64_t
  * (inference/int64_gemm.cu:708,729 and :629,650).  0 (default): R is left untouched. */
 void zk_softmax_clobber_input(int on);
 
+/* Fusion around the softmax (no counterpart in the reference's library; it replaces the tensor ops of
+ * inference/model.py:896-906 and the softmax_q19 call of :908-915 by one pass):
+ *   x = floor((s1 + s2) * mul / div) + mask[s][t];   scores = x (if not null);   C = softmax_q19(x)
+ * s1, s2 (may be null), scores (may be null), C: [Bsz,S,H,T]; mask (may be null): [S,T] broadcast over batch and
+ * heads; 0 < div < 2^31; arithmetic wraps like torch's int64 ops; the floor division is torch's `//`.
+ * Rows longer than 2048 need the scores buffer. */
+void softmax_q19_scores(const int64_t *s1, const int64_t *s2, const int64_t *mask, int64_t *scores, int64_t *C,
+                        const int64_t *lut, int Bsz, int S, int H, int T, int64_t mul, int64_t div);
+
+/* Fusion around the SiLU of the FFNs (no counterpart in the reference's library; it replaces silu_q23 plus the
+ * tensor ops of inference/model.py:1039-1048 and :1271-1280):  C = (silu_q23(R) * U) >> 23 with a wrapping product;
+ * the SiLU values themselves are stored to S when S is not null.  All tensors [Bsz,S,Dim]. */
+void silu_mul_q23(const int64_t *R, const int64_t *U, int64_t *S, int64_t *C, const int64_t *lut, int Bsz, int Sq, int Dim);
+
 /* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
 void zk_gemm_set_path(int path);

@@ -232,6 +232,26 @@ def sigmoid_q25(R, lut=None):
     return _act(_lib.ora_act_q25, R, silu_init_q25() if lut is None else lut, 1)
 
 
+def softmax_q19_scores(s1, s2, mask, mul=94, div=695, lut=None):
+    """(scores, C) of the fused call: the tensor ops of inference/model.py:896-906 restated with numpy's wrapping int64
+    arithmetic and floor division (what torch's `*`, `+` and `//` do), then softmax_q19 (:908-915)."""
+    with np.errstate(over="ignore"):
+        x = _c(s1).copy()
+        if s2 is not None:
+            x = x + _c(s2)
+        x = (x * np.int64(mul)) // np.int64(div)
+        if mask is not None:
+            x = x + _c(mask)[None, :, None, :]
+    return x, softmax_q19(x, lut)[0]
+
+
+def silu_mul_q23(R, U, lut=None):
+    """(silu, C) of the fused call: silu_q23, then the wrapping product and the floor shift of inference/model.py:1048"""
+    s = silu_q23(R, lut)
+    with np.errstate(over="ignore"):
+        return s, (s * _c(U)) >> 23
+
+
 def bf16_to_int32_2d(bits, rescale):
     """bits: uint16 bf16 patterns [rows, cols] -> int32 fixed point (inference/int64_gemm.cu:92-132)"""
     bits = _c(bits, np.uint16)

@@ -32,6 +32,16 @@ class CpuBackend:
     def rmsnorm(self, x2d, w, dim):
         return self.o.RMS_Norm_int64(x2d, w, 1, dim)[0]
 
+    def softmax_scores(self, s1, s2, mask):
+        """(scores, probabilities): inference/model.py:896-915 as the reference writes it, op by op"""
+        scores = (s1 + s2) * 94 // 695           # floor division (model.py:897)
+        if mask is not None:
+            scores = scores + mask[:, None, :]   # mask.unsqueeze(1) (model.py:905)
+        return scores, self.softmax(scores)
+
+    def silu_mul(self, r1, r2):
+        return (self.silu(r1) * r2) >> 23        # model.py:1048 uses // 2^23, :1280 uses >> 23: the same floor
+
     def rope(self, x, table):
         return self.o.complex_int64_mul_broadcast(x, table)
 
@@ -86,6 +96,9 @@ class GpuBackend:
     def rmsnorm(self, x2d, w, dim):
         return self.k.RMS_Norm_int64(x2d.contiguous(), w, 1, dim)[0]
 
+    softmax_scores = CpuBackend.softmax_scores   # the same op-by-op chain, on torch tensors
+    silu_mul = CpuBackend.silu_mul
+
     def rope(self, x, table):
         return self.k.complex_int64_mul_broadcast(x.contiguous(), table.contiguous())
 
@@ -107,6 +120,20 @@ class GpuBackend:
     def index_add_rows(self, y, idx, v):
         y.index_add_(0, idx, v)
         return y
+
+
+class FusedGpuBackend(GpuBackend):
+    """GpuBackend that takes the library's fused entry points where the reference chains tensor ops around a kernel"""
+
+    def softmax_scores(self, s1, s2, mask):
+        scores, p = self.t.empty_like(s1), self.t.empty_like(s1)
+        self.k.softmax_q19_scores(s1.contiguous(), s2.contiguous(), None if mask is None else mask.contiguous(), p, scores)
+        return scores, p
+
+    def silu_mul(self, r1, r2):
+        out = self.t.empty_like(r1)
+        self.k.silu_mul_q23(r1.contiguous(), r2.contiguous(), out)
+        return out
 
 
 class CheckedGpuBackend(GpuBackend):
@@ -200,8 +227,7 @@ def expert_ffn(be, x, w1, w2, w3, c13, c2):
     (inference/model.py:1018-1049, 1247-1281).  x [1,M,dim] Q23 activations."""
     r1, _ = be.linear(x, w1, c13)
     r2, _ = be.linear(x, w3, c13)
-    s1 = be.silu(r1)
-    h = (s1 * r2) >> 23                     # model.py:1048 uses // 2^23, :1280 uses >> 23: the same floor
+    h = be.silu_mul(r1, r2)
     y, _ = be.linear(h, w2, c2)
     return y
 
@@ -211,12 +237,7 @@ def attention_scores_softmax_pv(be, q_nope, q_pe, kv_cache, pe_cache, causal=Tru
     (inference/model.py:884-936).  q_nope [1,S,H,C], q_pe [1,S,H,R], kv_cache [1,T,C], pe_cache [1,T,R]."""
     s1 = be.einsum("einsum_bshc_btc_bsht", q_nope, kv_cache, 23)
     s2 = be.einsum("einsum_bshc_btc_bsht", q_pe, pe_cache, 21)
-    scores = (s1 + s2) * 94 // 695           # floor division (model.py:897)
-    if causal:
-        S, T = scores.shape[1], scores.shape[3]
-        m = be.causal_mask(S, T)
-        scores = scores + m[:, None, :]      # mask.unsqueeze(1) (model.py:905)
-    p = be.softmax(scores)
+    scores, p = be.softmax_scores(s1, s2, be.causal_mask(s1.shape[1], s1.shape[3]) if causal else None)
     out = be.einsum("einsum_bsht_btc_bshc", p, kv_cache, 23)
     return scores, p, out
 

@@ -498,6 +498,62 @@ def test_activation_table_path(K, oracle, fn, Q):
     oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("T", [1, 7, 64, 100, 1024, 2048, 2050, 3001])
+@pytest.mark.parametrize("with_s2,with_mask,keep_scores", [(True, True, True), (False, False, False), (True, False, True), (False, True, False)])
+def test_softmax_q19_scores_fusion(K, oracle, T, with_s2, with_mask, keep_scores):
+    """fused score preparation + softmax against the op-by-op restatement (inference/model.py:896-915)"""
+    if T > 2048 and not keep_scores:
+        pytest.skip("rows longer than 2048 need the scores buffer")
+    rng = np.random.default_rng(T * 8 + with_s2 * 4 + with_mask * 2 + keep_scores)
+    shape = (2, 3, 5, T)
+    s1 = rng.integers(-(40 << 19), 40 << 19, size=shape, dtype=np.int64)
+    s2 = rng.integers(-(40 << 19), 40 << 19, size=shape, dtype=np.int64) if with_s2 else None
+    s1.ravel()[:3] = [(1 << 62) + 12345, -(1 << 62) - 999, -1]        # the multiplication by 94 wraps, as in torch
+    mask = np.triu(np.full((3, T), -(64 << 36), np.int64), 1) if with_mask else None
+    C = torch.empty(shape, dtype=torch.int64, device="cuda")
+    scores = torch.empty(shape, dtype=torch.int64, device="cuda") if keep_scores else None
+    K.softmax_q19_scores(dev(s1), None if s2 is None else dev(s2), None if mask is None else dev(mask), C, scores)
+    xe, Ce = oracle.softmax_q19_scores(s1, s2, mask)
+    if keep_scores:
+        assert np.array_equal(host(scores), xe)
+    assert np.array_equal(host(C), Ce)
+
+
+def test_softmax_q19_scores_other_divisors_and_alignment(K, oracle):
+    rng = np.random.default_rng(5)
+    shape = (1, 4, 2, 129)
+    s1 = rng.integers(-(1 << 40), 1 << 40, size=shape, dtype=np.int64)
+    s2 = rng.integers(-(1 << 40), 1 << 40, size=shape, dtype=np.int64)
+    for mul, div in ((1, 1), (-3, 7), (94, 695), (12345, (1 << 31) - 1)):
+        C = torch.empty(shape, dtype=torch.int64, device="cuda")
+        sc = torch.empty(shape, dtype=torch.int64, device="cuda")
+        K.softmax_q19_scores(dev(s1), dev(s2), None, C, sc, mul=mul, div=div)
+        xe, Ce = oracle.softmax_q19_scores(s1, s2, None, mul, div)
+        assert np.array_equal(host(sc), xe), (mul, div)
+        assert np.array_equal(host(C), Ce), (mul, div)
+    with pytest.raises(RuntimeError):
+        K.softmax_q19_scores(dev(s1), dev(s2), None, C, sc, div=0)
+    K.lib.zk_clear_error()
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (1, 3, 7), (2, 5, 129), (1, 64, 2048), (1, 600, 2048)])
+@pytest.mark.parametrize("keep", [False, True])
+def test_silu_mul_q23_fusion(K, oracle, shape, keep):
+    """fused SiLU gate product against silu_q23 followed by the reference's tensor ops (inference/model.py:1039-1048);
+    the largest shape takes the quotient-table kernel"""
+    rng = np.random.default_rng(sum(shape) + keep)
+    r = rng.integers(-(20 << 23), 20 << 23, size=shape, dtype=np.int64)
+    u = rng.integers(-(1 << 45), 1 << 45, size=shape, dtype=np.int64)
+    r.ravel()[0] = 70 << 23                                          # the pass-through branch: silu(x) = x
+    C = torch.empty(shape, dtype=torch.int64, device="cuda")
+    S = torch.empty(shape, dtype=torch.int64, device="cuda") if keep else None
+    K.silu_mul_q23(dev(r), dev(u), C, S)
+    se, ce = oracle.silu_mul_q23(r, u)
+    assert np.array_equal(host(C), ce)
+    if keep:
+        assert np.array_equal(host(S), se)
+
+
 def test_converters(K, oracle):
     """the three float -> fixed converters the reference exports (inference/int64_gemm.cu:92-221)"""
     rng = np.random.default_rng(31)

@@ -67,9 +67,16 @@ __device__ __forceinline__ int64_t act_one(int64_t r, const int64_t *lut)
 constexpr int kActThreads = 256;
 constexpr int kActUnroll = 4;
 
-template <int Q, bool SIGMOID, bool VEC>
+// GATED (SiLU only): C = (silu(R) * U) >> Q, the gate product of the FFNs (inference/model.py:1048, :1280), and
+// the SiLU values themselves go to S when it is not null (the witness dump keeps them, model.py:1037-1042).
+struct ActGate { const int64_t *U; int64_t *S; };
+
+template <int Q>
+__device__ __forceinline__ int64_t gate_mul(int64_t s, int64_t u) { return (int64_t)((uint64_t)s * (uint64_t)u) >> Q; }
+
+template <int Q, bool SIGMOID, bool VEC, bool GATED>
 __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restrict__ R, int64_t *__restrict__ C,
-                                                          const int64_t *__restrict__ lut_g, long n)
+                                                          const int64_t *__restrict__ lut_g, long n, ActGate gate)
 {
     __shared__ int64_t lut[256];
     lut[threadIdx.x] = lut_g[threadIdx.x];
@@ -77,11 +84,14 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
     if (VEC) {
         long nvec = n >> 1;
         long base = (long)blockIdx.x * (kActThreads * kActUnroll) + threadIdx.x;
-        i64x2 v[kActUnroll];
+        i64x2 v[kActUnroll], u[GATED ? kActUnroll : 1];
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
             long i = base + (long)j * kActThreads;
-            if (i < nvec) v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
+            if (i < nvec) {
+                v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
+                if (GATED) u[j] = ld_stream(reinterpret_cast<const i64x2 *>(gate.U) + i);
+            }
         }
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
@@ -90,16 +100,29 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
                 i64x2 o;
                 o.x = act_one<Q, SIGMOID>(v[j].x, lut);
                 o.y = act_one<Q, SIGMOID>(v[j].y, lut);
+                if (GATED) {
+                    if (gate.S) st_stream(reinterpret_cast<i64x2 *>(gate.S) + i, o);
+                    o.x = gate_mul<Q>(o.x, u[j].x);
+                    o.y = gate_mul<Q>(o.y, u[j].y);
+                }
                 st_stream(reinterpret_cast<i64x2 *>(C) + i, o);
             }
         }
-        if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) C[n - 1] = act_one<Q, SIGMOID>(R[n - 1], lut);
+        if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) {
+            int64_t o = act_one<Q, SIGMOID>(R[n - 1], lut);
+            if (GATED) { if (gate.S) gate.S[n - 1] = o; o = gate_mul<Q>(o, gate.U[n - 1]); }
+            C[n - 1] = o;
+        }
     } else {
         long base = (long)blockIdx.x * (kActThreads * kActUnroll) + threadIdx.x;
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
             long i = base + (long)j * kActThreads;
-            if (i < n) C[i] = act_one<Q, SIGMOID>(R[i], lut);
+            if (i < n) {
+                int64_t o = act_one<Q, SIGMOID>(R[i], lut);
+                if (GATED) { if (gate.S) gate.S[i] = o; o = gate_mul<Q>(o, gate.U[i]); }
+                C[i] = o;
+            }
         }
     }
 }
@@ -134,11 +157,11 @@ __global__ __launch_bounds__(256) void act_qtab_kernel(const int64_t *__restrict
 
 constexpr int kTabThreads = 512;
 
-template <int Q, bool SIGMOID>
+template <int Q, bool SIGMOID, bool GATED>
 __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *__restrict__ R, int64_t *__restrict__ C,
                                                                 const int64_t *__restrict__ lut_g,
                                                                 const uint32_t *__restrict__ qtab_g,
-                                                                const int *__restrict__ ok_g, long n)
+                                                                const int *__restrict__ ok_g, long n, ActGate gate)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char act_smem[];
     int64_t *lut = reinterpret_cast<int64_t *>(act_smem);
@@ -174,11 +197,14 @@ __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *_
     const long nvec = n >> 1;
     const long stride = (long)gridDim.x * (kTabThreads * kActUnroll);
     for (long base = (long)blockIdx.x * (kTabThreads * kActUnroll) + threadIdx.x; base < nvec; base += stride) {
-        i64x2 v[kActUnroll];
+        i64x2 v[kActUnroll], u[GATED ? kActUnroll : 1];
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
             long i = base + (long)j * kTabThreads;
-            if (i < nvec) v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
+            if (i < nvec) {
+                v[j] = ld_stream(reinterpret_cast<const i64x2 *>(R) + i);
+                if (GATED) u[j] = ld_stream(reinterpret_cast<const i64x2 *>(gate.U) + i);
+            }
         }
 #pragma unroll
         for (int j = 0; j < kActUnroll; j++) {
@@ -187,25 +213,35 @@ __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *_
                 i64x2 o;
                 o.x = one(v[j].x);
                 o.y = one(v[j].y);
+                if (GATED) {
+                    if (gate.S) st_stream(reinterpret_cast<i64x2 *>(gate.S) + i, o);
+                    o.x = gate_mul<Q>(o.x, u[j].x);
+                    o.y = gate_mul<Q>(o.y, u[j].y);
+                }
                 st_stream(reinterpret_cast<i64x2 *>(C) + i, o);
             }
         }
     }
-    if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) C[n - 1] = one(R[n - 1]);
+    if ((n & 1) && blockIdx.x == 0 && threadIdx.x == 0) {
+        int64_t o = one(R[n - 1]);
+        if (GATED) { if (gate.S) gate.S[n - 1] = o; o = gate_mul<Q>(o, gate.U[n - 1]); }
+        C[n - 1] = o;
+    }
 }
 
 static uint32_t *g_qtab = nullptr;      // (2Q+2)*256 quotients + the ok flag behind them, kept for the process lifetime
 constexpr size_t kQtabBytes = (size_t)QTab<25>::kEntries * 4;
 constexpr size_t kQtabFlagBytes = (size_t)QTab<25>::kRows * 4;
 
-template <int Q, bool SIGMOID>
-static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim)
+template <int Q, bool SIGMOID, bool GATED = false>
+static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim,
+                       ActGate gate = ActGate{ nullptr, nullptr })
 {
     if (Bsz < 0 || S < 0 || Dim < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
     long n = (long)Bsz * S * Dim;
     if (n == 0) return;
-    if (!R || !C || !lut) { set_error(kBadArgument, "%s: null pointer", name); return; }
-    bool vec = (((uintptr_t)R | (uintptr_t)C) & 15) == 0;
+    if (!R || !C || !lut || (GATED && !gate.U)) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    bool vec = (((uintptr_t)R | (uintptr_t)C | (uintptr_t)gate.U | (uintptr_t)gate.S) & 15) == 0;
     if (vec && n >= (1L << 20)) {
         if (!g_qtab && hipMalloc(&g_qtab, kQtabBytes + kQtabFlagBytes) != hipSuccess) {
             (void)hipGetLastError();
@@ -217,7 +253,7 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
             const size_t lds = 2048 + (size_t)QTab<Q>::kEntries * 4;
             static bool raised = false;
             if (!raised) {
-                if (hipFuncSetAttribute((const void *)act_table_kernel<Q, SIGMOID>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                if (hipFuncSetAttribute((const void *)act_table_kernel<Q, SIGMOID, GATED>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)lds) != hipSuccess) {
                     set_error(kLaunchFailure, "%s: cannot raise the LDS limit", name);
                     return;
@@ -227,7 +263,7 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
             const long per_block = (long)kTabThreads * kActUnroll;
             long blocks = ((n >> 1) + per_block - 1) / per_block;
             if (blocks > 512) blocks = 512;            // persistent (2 per CU): each workgroup loads the table once
-            act_table_kernel<Q, SIGMOID><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, n);
+            act_table_kernel<Q, SIGMOID, GATED><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, n, gate);
             check_launch(name);
             return;
         }
@@ -235,8 +271,8 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
     long per_block = (long)kActThreads * kActUnroll;
     long items = vec ? ((n >> 1) > 0 ? (n >> 1) : 1) : n;
     long blocks = (items + per_block - 1) / per_block;
-    if (vec) act_kernel<Q, SIGMOID, true><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n);
-    else act_kernel<Q, SIGMOID, false><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n);
+    if (vec) act_kernel<Q, SIGMOID, true, GATED><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n, gate);
+    else act_kernel<Q, SIGMOID, false, GATED><<<dim3((unsigned)blocks), dim3(kActThreads), 0, 0>>>(R, C, lut, n, gate);
     check_launch(name);
 }
 
@@ -392,6 +428,11 @@ void silu_q25(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
 void sigmoid_q25(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int Dim)
 {
     zk::launch_act<25, true>("sigmoid_q25", R, C, lut, Bsz, S, Dim);
+}
+
+void silu_mul_q23(const int64_t *R, const int64_t *U, int64_t *S, int64_t *C, const int64_t *lut, int Bsz, int Sq, int Dim)
+{
+    zk::launch_act<23, false, true>("silu_mul_q23", R, C, lut, Bsz, Sq, Dim, zk::ActGate{ U, S });
 }
 
 void complex_int64_mul(const int64_t *A, const int64_t *B, int64_t *C, int batchSize, int seqLen, int headCount,

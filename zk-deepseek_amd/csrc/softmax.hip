@@ -70,11 +70,67 @@ __device__ __forceinline__ int64_t smx_norm(int64_t w, int64_t s, double inv, bo
 
 constexpr int kSmxThreads = 256;
 
+// Optional score preparation fused into the row load (inference/model.py:896-906 does it with three tensor ops):
+//   x = floor((s1 + s2) * mul / div) + mask[s][t]
+// s2, mask and scores (a copy of x for the witness dump, model.py:911-918) may be null.
+struct SmxPre {
+    const int64_t *s2;
+    const int64_t *mask;      // [S, T], added to every batch and head
+    int64_t *scores;
+    int64_t mul, div;
+    double inv_div;
+    int S, H;
+};
+
+// floor(x / d) for 0 < d < 2^31 and any x: double estimate (exact to within one for |x| < 2^62, within a few
+// otherwise) settled by the remainder
+__device__ __forceinline__ int64_t floordiv_small(int64_t x, int64_t d, double inv_d)
+{
+    int64_t q = (int64_t)floor((double)x * inv_d);
+    int64_t rem = (int64_t)((uint64_t)x - (uint64_t)q * (uint64_t)d);
+    while (rem < 0) { q--; rem += d; }
+    while (rem >= d) { q++; rem -= d; }
+    return q;
+}
+
+__device__ __forceinline__ int64_t smx_prepare_value(int64_t v, int64_t s2, int64_t m, const SmxPre &pre)
+{
+    v = (int64_t)((uint64_t)v + (uint64_t)s2);
+    v = (int64_t)((uint64_t)v * (uint64_t)pre.mul);
+    if (pre.div != 1) v = floordiv_small(v, pre.div, pre.inv_div);
+    return (int64_t)((uint64_t)v + (uint64_t)m);
+}
+
+template <bool PRE>
+__device__ __forceinline__ int64_t smx_prepare(int64_t v, const SmxPre &pre, long row, int idx, int T)
+{
+    if (!PRE) return v;
+    const long e = row * T + idx;
+    v = smx_prepare_value(v, pre.s2 ? pre.s2[e] : 0, pre.mask ? pre.mask[(long)((row / pre.H) % pre.S) * T + idx] : 0, pre);
+    if (pre.scores) pre.scores[e] = v;
+    return v;
+}
+
+// two adjacent elements at once, every access 16 bytes wide (the caller has checked the alignment)
+template <bool PRE>
+__device__ __forceinline__ i64x2s smx_prepare_pair(i64x2s p, const SmxPre &pre, long row, int idx, int T)
+{
+    if (!PRE) return p;
+    const long e = row * T + idx;
+    i64x2s b = { 0, 0 }, m = { 0, 0 };
+    if (pre.s2) b = ld_stream(reinterpret_cast<const i64x2s *>(pre.s2 + e));
+    if (pre.mask) m = *reinterpret_cast<const i64x2s *>(pre.mask + (long)((row / pre.H) % pre.S) * T + idx);
+    p.x = smx_prepare_value(p.x, b.x, m.x, pre);
+    p.y = smx_prepare_value(p.y, b.y, m.y, pre);
+    if (pre.scores) st_stream(reinterpret_cast<i64x2s *>(pre.scores + e), p);
+    return p;
+}
+
 // One row per wavefront; EPL = elements per lane (even).  VEC: T is even and the pointers are 16-byte aligned.
-template <int Q, int EPL, bool VEC>
+template <int Q, int EPL, bool VEC, bool PRE>
 __global__ __launch_bounds__(kSmxThreads) void softmax_wave_kernel(int64_t *__restrict__ R, int64_t *__restrict__ C,
                                                                    const int64_t *__restrict__ lut_g, long rows, int T,
-                                                                   int clobber)
+                                                                   int clobber, SmxPre pre)
 {
     __shared__ int64_t lut[256];
     lut[threadIdx.x] = lut_g[threadIdx.x];
@@ -93,14 +149,15 @@ __global__ __launch_bounds__(kSmxThreads) void softmax_wave_kernel(int64_t *__re
         if (VEC) {
             if (idx < T) {
                 i64x2s p = ld_stream(reinterpret_cast<const i64x2s *>(x + idx));
+                p = smx_prepare_pair<PRE>(p, pre, row, idx, T);
                 v[2 * j] = p.x;
                 v[2 * j + 1] = p.y;
                 rmax = p.x > rmax ? p.x : rmax;
                 rmax = p.y > rmax ? p.y : rmax;
             }
         } else {
-            if (idx < T) { v[2 * j] = x[idx]; rmax = v[2 * j] > rmax ? v[2 * j] : rmax; }
-            if (idx + 1 < T) { v[2 * j + 1] = x[idx + 1]; rmax = v[2 * j + 1] > rmax ? v[2 * j + 1] : rmax; }
+            if (idx < T) { v[2 * j] = smx_prepare<PRE>(x[idx], pre, row, idx, T); rmax = v[2 * j] > rmax ? v[2 * j] : rmax; }
+            if (idx + 1 < T) { v[2 * j + 1] = smx_prepare<PRE>(x[idx + 1], pre, row, idx + 1, T); rmax = v[2 * j + 1] > rmax ? v[2 * j + 1] : rmax; }
         }
     }
     rmax = wave_max_i64(rmax);
@@ -188,31 +245,58 @@ __global__ __launch_bounds__(kSmxThreads) void softmax_block_kernel(int64_t *__r
 }
 
 template <int Q, int EPL>
-static void launch_wave(int64_t *R, int64_t *C, const int64_t *lut, long rows, int T, bool vec, int clobber)
+static void launch_wave(int64_t *R, int64_t *C, const int64_t *lut, long rows, int T, bool vec, int clobber, const SmxPre *pre)
 {
     long blocks = (rows + (kSmxThreads / 64) - 1) / (kSmxThreads / 64);
-    if (vec)
-        softmax_wave_kernel<Q, EPL, true><<<dim3((unsigned)blocks), dim3(kSmxThreads), 0, 0>>>(R, C, lut, rows, T, clobber);
-    else
-        softmax_wave_kernel<Q, EPL, false><<<dim3((unsigned)blocks), dim3(kSmxThreads), 0, 0>>>(R, C, lut, rows, T, clobber);
+    const dim3 grid((unsigned)blocks), block(kSmxThreads);
+    SmxPre none = {};
+    if (pre) {
+        if (vec) softmax_wave_kernel<Q, EPL, true, true><<<grid, block, 0, 0>>>(R, C, lut, rows, T, clobber, *pre);
+        else softmax_wave_kernel<Q, EPL, false, true><<<grid, block, 0, 0>>>(R, C, lut, rows, T, clobber, *pre);
+    } else {
+        if (vec) softmax_wave_kernel<Q, EPL, true, false><<<grid, block, 0, 0>>>(R, C, lut, rows, T, clobber, none);
+        else softmax_wave_kernel<Q, EPL, false, false><<<grid, block, 0, 0>>>(R, C, lut, rows, T, clobber, none);
+    }
+}
+
+// the score preparation as a pass of its own, for rows too long for the one-row-per-wavefront kernel
+__global__ __launch_bounds__(256) void smx_prepare_kernel(const int64_t *__restrict__ s1, int64_t *__restrict__ out, long rows, int T, SmxPre pre)
+{
+    const long e = (long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= rows * T) return;
+    SmxPre q = pre;
+    q.scores = nullptr;
+    out[e] = smx_prepare<true>(s1[e], q, e / T, (int)(e % T), T);
 }
 
 template <int Q>
-static void launch_softmax(const char *name, int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int H, int T)
+static void launch_softmax(const char *name, int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int H, int T,
+                           const SmxPre *pre = nullptr)
 {
     if (Bsz < 0 || S < 0 || H < 0 || T < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
     long rows = (long)Bsz * S * H;
     if (rows == 0 || T == 0) return;
     if (!R || !C || !lut) { set_error(kBadArgument, "%s: null pointer", name); return; }
     if (rows > 0x7FFFFFFFL) { set_error(kUnsupportedSize, "%s: more than 2^31-1 rows", name); return; }
-    int clobber = g_softmax_clobber ? 1 : 0;
+    int clobber = g_softmax_clobber && !pre ? 1 : 0;
     bool vec = (T % 2 == 0) && ((((uintptr_t)R | (uintptr_t)C) & 15) == 0);
-    if (T <= 128) launch_wave<Q, 2>(R, C, lut, rows, T, vec, clobber);
-    else if (T <= 256) launch_wave<Q, 4>(R, C, lut, rows, T, vec, clobber);
-    else if (T <= 512) launch_wave<Q, 8>(R, C, lut, rows, T, vec, clobber);
-    else if (T <= 1024) launch_wave<Q, 16>(R, C, lut, rows, T, vec, clobber);
-    else if (T <= 2048) launch_wave<Q, 32>(R, C, lut, rows, T, vec, clobber);
-    else softmax_block_kernel<Q><<<dim3((unsigned)rows), dim3(kSmxThreads), 0, 0>>>(R, C, lut, T, clobber);
+    if (pre && ((((uintptr_t)pre->s2 | (uintptr_t)pre->mask | (uintptr_t)pre->scores) & 15) != 0)) vec = false;
+    if (T <= 128) launch_wave<Q, 2>(R, C, lut, rows, T, vec, clobber, pre);
+    else if (T <= 256) launch_wave<Q, 4>(R, C, lut, rows, T, vec, clobber, pre);
+    else if (T <= 512) launch_wave<Q, 8>(R, C, lut, rows, T, vec, clobber, pre);
+    else if (T <= 1024) launch_wave<Q, 16>(R, C, lut, rows, T, vec, clobber, pre);
+    else if (T <= 2048) launch_wave<Q, 32>(R, C, lut, rows, T, vec, clobber, pre);
+    else {
+        if (pre) {
+            // long rows: prepared scores go to the scores buffer if there is one, else through C (the block kernel
+            // reads all of a row before it writes any of it only when input and output differ, so C cannot serve as both)
+            if (!pre->scores) { set_error(kBadArgument, "%s: rows longer than 2048 need a scores buffer", name); return; }
+            const long n = rows * T;
+            smx_prepare_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(R, pre->scores, rows, T, *pre);
+            R = pre->scores;
+        }
+        softmax_block_kernel<Q><<<dim3((unsigned)rows), dim3(kSmxThreads), 0, 0>>>(R, C, lut, T, clobber);
+    }
     check_launch(name);
 }
 
@@ -231,5 +315,16 @@ void softmax_q21(int64_t *R, int64_t *C, int64_t *lut, int Bsz, int S, int H, in
 }
 
 void zk_softmax_clobber_input(int on) { zk::g_softmax_clobber = on != 0; }
+
+void softmax_q19_scores(const int64_t *s1, const int64_t *s2, const int64_t *mask, int64_t *scores, int64_t *C,
+                        const int64_t *lut, int Bsz, int S, int H, int T, int64_t mul, int64_t div)
+{
+    const char *name = "softmax_q19_scores";
+    if (div <= 0 || div >= ((int64_t)1 << 31)) { zk::set_error(zk::kBadArgument, "%s: div must be in [1, 2^31)", name); return; }
+    zk::SmxPre pre;
+    pre.s2 = s2; pre.mask = mask; pre.scores = scores; pre.mul = mul; pre.div = div; pre.inv_div = 1.0 / (double)div;
+    pre.S = S > 0 ? S : 1; pre.H = H > 0 ? H : 1;
+    zk::launch_softmax<19>(name, const_cast<int64_t *>(s1), C, lut, Bsz, S, H, T, &pre);
+}
 
 }  // extern "C"

@@ -65,6 +65,8 @@ lib.zk_gemm_get_path.restype = _ci
 lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
 lib.zk_timer_stop_ms.restype = ctypes.c_float
 lib.zk_gemm_guard_hits.restype = ctypes.c_long
+lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
+lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
 lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
 
@@ -298,3 +300,30 @@ def silu_q23(R: torch.Tensor, C: torch.Tensor):
 
 def sigmoid_q23(R: torch.Tensor, C: torch.Tensor):
     _act(lib.sigmoid_q23, "sigmoid_q23", R, C, EXP2_FRAC_LUT_Q23)
+
+
+# ---- fusions (no counterpart in the reference's kernel.py: each replaces a kernel call plus the tensor ops around it)
+def softmax_q19_scores(s1, s2, mask, C, scores=None, mul=94, div=695):
+    """C = softmax_q19(floor((s1 + s2) * mul / div) + mask[None, :, None, :]) in one pass over [Bsz,S,H,T]; the
+    prepared scores are also written to `scores` when given (inference/model.py:896-915).  s2 and mask may be None."""
+    assert s1.is_cuda and C.is_cuda and s1.dtype == torch.int64 and s1.is_contiguous() and C.is_contiguous()
+    assert EXP2_FRAC_LUT_Q19 is not None, "call softmax_init_q19 first"
+    Bsz, S, H, T = s1.shape
+    for t in (s2, scores):
+        assert t is None or (t.is_cuda and t.dtype == torch.int64 and t.is_contiguous() and tuple(t.shape) == (Bsz, S, H, T))
+    assert mask is None or (mask.is_cuda and mask.dtype == torch.int64 and mask.is_contiguous() and tuple(mask.shape) == (S, T))
+    ptr = lambda t: 0 if t is None else t.data_ptr()
+    lib.softmax_q19_scores(s1.data_ptr(), ptr(s2), ptr(mask), ptr(scores), C.data_ptr(), EXP2_FRAC_LUT_Q19.data_ptr(),
+                           Bsz, S, H, T, int(mul), int(div))
+    _check("softmax_q19_scores")
+
+
+def silu_mul_q23(R, U, C, S=None):
+    """C = (silu_q23(R) * U) >> 23 in one pass; the SiLU values go to S when given (inference/model.py:1039-1048)."""
+    assert R.is_cuda and U.is_cuda and C.is_cuda and R.shape == U.shape == C.shape
+    assert R.is_contiguous() and U.is_contiguous() and C.is_contiguous() and (S is None or S.is_contiguous())
+    assert EXP2_FRAC_LUT_Q23 is not None, "call silu_init_q23 first"
+    Bsz, Sq, Dim = R.shape
+    lib.silu_mul_q23(R.data_ptr(), U.data_ptr(), 0 if S is None else S.data_ptr(), C.data_ptr(),
+                     EXP2_FRAC_LUT_Q23.data_ptr(), Bsz, Sq, Dim)
+    _check("silu_mul_q23")
