@@ -243,6 +243,14 @@ def main():
         extra["silu_mul_q23_fused_1x8192x18432_24B_per_element"]["unfused_chain_ms"] = timed(K, chain2, 5, 2)
         del r1, r2, hh
 
+        # expert routing of the gate: 256 experts in 8 groups, 4 groups kept, top 8 (8*256 + 2*8*8 bytes per token)
+        gr = torch.Generator(device="cpu").manual_seed(800)
+        gbias = randint(gr, -(1 << 18), 1 << 18, (256,)).to(torch.int32).cuda()
+        for Tt in (256, 65536):
+            gsc = randint(gr, 1, 1 << 23, (Tt, 256)).cuda()
+            hbm("gate_route_%dx256" % Tt, lambda: K.gate_route(gsc, gbias, 8, 4, 8), Tt, bytes_per_elem=8.0 * 256 + 128.0, steps=20)
+            del gsc
+
         # RoPE and the float -> fixed converters (weight-loading path), by their own algorithmic bytes per element
         gq = torch.Generator(device="cpu").manual_seed(700)
         q_pe = randint(gq, -(1 << 30), 1 << 30, (1, 4096, 128, 32, 2)).cuda()

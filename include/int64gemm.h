@@ -128,6 +128,16 @@ void softmax_q19_scores(const int64_t *s1, const int64_t *s2, const int64_t *mas
  * the SiLU values themselves are stored to S when S is not null.  All tensors [Bsz,S,Dim]. */
 void silu_mul_q23(const int64_t *R, const int64_t *U, int64_t *S, int64_t *C, const int64_t *lut, int Bsz, int Sq, int Dim);
 
+/* Expert routing of the MoE gate (no counterpart in the reference's library; it replaces the tensor ops of
+ * Gate.forward, inference/model.py:1143-1208, on the output of sigmoid_q23).  scores [T,E] int64 (Q23), bias [E]
+ * int32 or null.  Per token: biased scores; each of the n_groups groups scored by the sum of its two largest biased
+ * scores (its maximum without bias); the topk_groups best groups kept, the others count as -2^42; the topk largest
+ * biased scores win, in descending order, ties to the lower index (torch.topk leaves ties to its implementation).
+ * indices [T,topk] int64; raw_weights [T,topk] (may be null) = the winners' UNBIASED scores (gate_weights.bin);
+ * weights [T,topk] = floor(floor(raw * 2^23 / sum raw) * 5 / 2).  E <= 1024, n_groups <= 64 dividing E, topk <= 64. */
+void gate_route_q23(const int64_t *scores, const int32_t *bias, int64_t *weights, int64_t *indices,
+                    int64_t *raw_weights, int T, int E, int n_groups, int topk_groups, int topk);
+
 /* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
 void zk_gemm_set_path(int path);

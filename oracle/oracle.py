@@ -50,6 +50,7 @@ def _load():
         getattr(lib, name).argtypes = [vp, vp, vp, cl, ci]
     lib.ora_bf16_to_int32.argtypes = [vp, vp, cl, ci, ci]
     lib.ora_float32_to_int64.argtypes = [vp, vp, cl, ci]
+    lib.ora_gate_route.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.ora_set_threads.argtypes = [ci]
     lib.ora_max_threads.restype = ci
     return lib
@@ -250,6 +251,20 @@ def silu_mul_q23(R, U, lut=None):
     s = silu_q23(R, lut)
     with np.errstate(over="ignore"):
         return s, (s * _c(U)) >> 23
+
+
+def gate_route(scores, bias, n_groups, topk_groups, topk):
+    """(weights, indices, raw_weights) of Gate.forward's routing (inference/model.py:1143-1208); scores [T,E] int64,
+    bias [E] int32 or None"""
+    scores = _c(scores)
+    T, E = scores.shape
+    assert E <= 1024 and n_groups <= 64 and E % n_groups == 0
+    w = np.empty((T, topk), np.int64)
+    idx = np.empty((T, topk), np.int64)
+    raw = np.empty((T, topk), np.int64)
+    b = None if bias is None else _c(bias, np.int32)
+    _lib.ora_gate_route(_p(scores), None if b is None else _p(b), _p(w), _p(idx), _p(raw), T, E, n_groups, topk_groups, topk)
+    return w, idx, raw
 
 
 def bf16_to_int32_2d(bits, rescale):

@@ -480,3 +480,72 @@ void ora_float32_to_int64(const uint32_t *in, int64_t *out, long n, int rescale)
         out[i] = v;
     }
 }
+
+/* ---- expert routing of the MoE gate ------------------------------------------------------------
+ * The tensor ops of Gate.forward after sigmoid_q23 (inference/model.py:1143-1208), per token:
+ *   s = scores + bias (:1149); group score = sum of the two largest s of the group (:1166), the maximum when
+ *   there is no bias (:1162); the topk_groups best groups are kept (:1172), every s of the others becomes -2^42
+ *   (:1185); indices = the topk largest s (:1189); raw = scores gathered at indices (:1194);
+ *   weights = (raw * 2^23) // sum(raw) (:1203), then * 5 // 2 (:1208), `//` being floor division.
+ * torch.topk returns its winners in descending order and leaves ties to its implementation: here the lower
+ * index wins (parity unpinned on ties; sigmoid scores plus a bias rarely tie).  sum(raw) == 0 gives 0. */
+static int64_t ora_floordiv(int64_t a, int64_t b)
+{
+    if (b == 0) return 0;
+    int64_t q = a / b;
+    if ((a % b != 0) && ((a < 0) != (b < 0))) q--;
+    return q;
+}
+
+void ora_gate_route(const int64_t *scores, const int32_t *bias, int64_t *weights, int64_t *indices, int64_t *raw,
+                    int T, int E, int n_groups, int topk_groups, int topk)
+{
+    const int64_t masked = -((int64_t)1 << 42);
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+    for (int t = 0; t < T; t++) {
+        int64_t s[1024];
+        char gone[1024], keep[64], used[64];
+        int64_t gs[64];
+        const int64_t *row = scores + (long)t * E;
+        for (int e = 0; e < E; e++) s[e] = (int64_t)((uint64_t)row[e] + (uint64_t)(int64_t)(bias ? bias[e] : 0));
+        if (n_groups > 1) {
+            const int gsize = E / n_groups;
+            for (int g = 0; g < n_groups; g++) {
+                int i1 = -1, i2 = -1;
+                for (int e = g * gsize; e < (g + 1) * gsize; e++)
+                    if (i1 < 0 || s[e] > s[i1]) i1 = e;
+                for (int e = g * gsize; e < (g + 1) * gsize; e++)
+                    if (e != i1 && (i2 < 0 || s[e] > s[i2])) i2 = e;
+                gs[g] = bias ? (int64_t)((uint64_t)s[i1] + (uint64_t)(i2 >= 0 ? s[i2] : 0)) : s[i1];
+                keep[g] = 0;
+                used[g] = 0;
+            }
+            for (int k = 0; k < topk_groups; k++) {
+                int best = -1;
+                for (int g = 0; g < n_groups; g++)
+                    if (!used[g] && (best < 0 || gs[g] > gs[best])) best = g;
+                used[best] = 1;
+                keep[best] = 1;
+            }
+            for (int e = 0; e < E; e++)
+                if (!keep[e / gsize]) s[e] = masked;
+        }
+        for (int e = 0; e < E; e++) gone[e] = 0;
+        int64_t sum = 0;
+        for (int k = 0; k < topk; k++) {
+            int best = -1;
+            for (int e = 0; e < E; e++)
+                if (!gone[e] && (best < 0 || s[e] > s[best])) best = e;
+            gone[best] = 1;
+            indices[(long)t * topk + k] = best;
+            weights[(long)t * topk + k] = row[best];
+            sum = (int64_t)((uint64_t)sum + (uint64_t)row[best]);
+        }
+        for (int k = 0; k < topk; k++) {
+            int64_t w = weights[(long)t * topk + k];
+            if (raw) raw[(long)t * topk + k] = w;
+            w = ora_floordiv((int64_t)((uint64_t)w << 23), sum);
+            weights[(long)t * topk + k] = ora_floordiv((int64_t)((uint64_t)w * 5u), 2);
+        }
+    }
+}

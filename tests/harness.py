@@ -135,6 +135,11 @@ class FusedGpuBackend(GpuBackend):
         self.k.silu_mul_q23(r1.contiguous(), r2.contiguous(), out)
         return out
 
+    def route(self, scores, bias_host, cfg):
+        bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
+        w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"])
+        return w.cpu().numpy(), idx.cpu().numpy()
+
 
 class CheckedGpuBackend(GpuBackend):
     """GpuBackend that checks every kernel call against the CPU oracle on the call's ACTUAL inputs: completely
@@ -294,7 +299,7 @@ def moe(be, x, P, cfg):
     """MoE.forward (inference/model.py:1325-1383): shared expert + top-k routed experts, weights Q23"""
     T = x.shape[1]
     sc = gate_scores(be, x, P, cfg)
-    w_host, idx_host = route(be.to_host(sc), P["gate_bias_host"], cfg)
+    w_host, idx_host = be.route(sc, P["gate_bias_host"], cfg) if hasattr(be, "route") else route(be.to_host(sc), P["gate_bias_host"], cfg)
     y = be.zeros_like(x[0])
     for e in range(cfg["experts"]):
         tok, slot = np.nonzero(idx_host == e)

@@ -554,6 +554,22 @@ def test_silu_mul_q23_fusion(K, oracle, shape, keep):
         assert np.array_equal(host(S), se)
 
 
+@pytest.mark.parametrize("E,G,KG,K_", [(256, 8, 4, 8), (16, 4, 2, 4), (64, 1, 1, 6), (96, 3, 3, 5), (512, 8, 3, 8), (1024, 16, 5, 64), (7, 1, 1, 7)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_gate_route(K, oracle, E, G, KG, K_, with_bias):
+    """routing of Gate.forward on the device against the oracle, ties included (coarse scores tie often)"""
+    rng = np.random.default_rng(E * 3 + G + with_bias)
+    for T, hi in ((1, 1 << 23), (77, 1 << 23), (300, 12)):
+        scores = rng.integers(1, hi, size=(T, E), dtype=np.int64)
+        bias = rng.integers(-(hi >> 3) - 1, (hi >> 3) + 1, size=E, dtype=np.int64).astype(np.int32) if with_bias else None
+        raw = torch.empty((T, K_), dtype=torch.int64, device="cuda")
+        w, idx = K.gate_route(dev(scores), None if bias is None else dev(bias), G, KG, K_, raw)
+        we, ie, re_ = oracle.gate_route(scores, bias, G, KG, K_)
+        assert np.array_equal(host(idx), ie), "indices"
+        assert np.array_equal(host(raw), re_), "gathered scores"
+        assert np.array_equal(host(w), we), "weights"
+
+
 def test_converters(K, oracle):
     """the three float -> fixed converters the reference exports (inference/int64_gemm.cu:92-221)"""
     rng = np.random.default_rng(31)

@@ -333,3 +333,54 @@ def test_converters_truncate_the_scaled_float(oracle):
             assert o == 0x7FFFFFFF                                 # saturates regardless of sign (:151-154)
         else:
             assert o == pl                                         # otherwise the rescale-25 conversion
+
+
+# ------------------------------------------------------------------------------ gate routing ---
+def _route_numpy(scores, bias, n_groups, topk_groups, topk):
+    """independent restatement with numpy's sorts (stable, so ties go to the lower index)"""
+    T, E = scores.shape
+    sc = scores + (0 if bias is None else bias.astype(np.int64)[None, :])
+    if n_groups > 1:
+        grp = sc.reshape(T, n_groups, E // n_groups)
+        srt = -np.sort(-grp, axis=-1)
+        gscore = srt[..., :2].sum(-1) if bias is not None else srt[..., 0]
+        gsel = np.argsort(-gscore, axis=-1, kind="stable")[:, :topk_groups]
+        keep = np.zeros((T, n_groups), bool)
+        np.put_along_axis(keep, gsel, True, axis=1)
+        sc = np.where(np.repeat(keep, E // n_groups, axis=1), sc, -(1 << 42))
+    idx = np.argsort(-sc, axis=-1, kind="stable")[:, :topk]
+    raw = np.take_along_axis(scores, idx, axis=1)
+    w = (raw * (1 << 23)) // raw.sum(-1, keepdims=True)
+    return w * 5 // 2, idx, raw
+
+
+@pytest.mark.parametrize("E,G,KG,K", [(256, 8, 4, 8), (16, 4, 2, 4), (64, 1, 1, 6), (96, 3, 3, 5), (512, 8, 3, 8)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_gate_route_matches_the_tensor_op_restatement(oracle, E, G, KG, K, with_bias):
+    rng = np.random.default_rng(E + G + with_bias)
+    scores = rng.integers(1, 1 << 23, size=(50, E), dtype=np.int64)            # sigmoid_q23 outputs
+    bias = rng.integers(-(1 << 20), 1 << 20, size=E, dtype=np.int64).astype(np.int32) if with_bias else None
+    w, idx, raw = oracle.gate_route(scores, bias, G, KG, K)
+    we, ie, re_ = _route_numpy(scores, bias, G, KG, K)
+    assert np.array_equal(idx, ie) and np.array_equal(raw, re_) and np.array_equal(w, we)
+    # what the arithmetic fixes: winners are distinct, sorted by biased score, and the weights are Q23 shares * 2.5
+    assert all(len(set(r)) == K for r in idx.tolist())
+    assert np.all(w >= 0) and np.all(w.sum(-1) <= (5 << 23) // 2) and np.all(w.sum(-1) > ((5 << 23) // 2) - 3 * K)
+
+
+def test_gate_route_hand_case_and_ties(oracle):
+    """8 experts in 4 groups of 2, keep 2 groups, pick 3.  Biased scores by group: (10,1) (7,7) (9,3) (7,7): group
+    scores 11, 14, 12, 14 -> groups 1 and 3 win (the tie between them does not matter), group 2 beats group 0 for
+    nothing.  Among experts 2,3,6,7 all biased scores are 7: the lower indices win."""
+    scores = np.array([[10, 1, 7, 7, 9, 3, 7, 7]], np.int64)
+    w, idx, raw = oracle.gate_route(scores, np.zeros(8, np.int32), 4, 2, 3)
+    assert idx.tolist() == [[2, 3, 6]] and raw.tolist() == [[7, 7, 7]]
+    assert w.tolist() == [[((7 << 23) // 21) * 5 // 2] * 3]
+    # the bias decides the routing but the weights come from the unbiased scores
+    bias = np.array([0, 0, 0, 0, 100, 100, 0, 0], np.int32)
+    w, idx, raw = oracle.gate_route(scores, bias, 4, 2, 3)
+    assert idx.tolist() == [[4, 5, 2]] and raw.tolist() == [[9, 3, 7]]
+    assert w.tolist() == [[((9 << 23) // 19) * 5 // 2, ((3 << 23) // 19) * 5 // 2, ((7 << 23) // 19) * 5 // 2]]
+    # without a bias a group is scored by its maximum: 10, 7, 9, 7 -> groups 0 and 2
+    w, idx, raw = oracle.gate_route(scores, None, 4, 2, 3)
+    assert idx.tolist() == [[0, 4, 5]]

@@ -67,6 +67,7 @@ lib.zk_timer_stop_ms.restype = ctypes.c_float
 lib.zk_gemm_guard_hits.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
+lib.gate_route_q23.argtypes = [_vp] * 5 + [_ci] * 5
 lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
 
@@ -316,6 +317,21 @@ def softmax_q19_scores(s1, s2, mask, C, scores=None, mul=94, div=695):
     lib.softmax_q19_scores(s1.data_ptr(), ptr(s2), ptr(mask), ptr(scores), C.data_ptr(), EXP2_FRAC_LUT_Q19.data_ptr(),
                            Bsz, S, H, T, int(mul), int(div))
     _check("softmax_q19_scores")
+
+
+def gate_route(scores, bias, n_groups, topk_groups, topk, raw_weights=None):
+    """Routing of Gate.forward on the device (inference/model.py:1143-1208): scores [T,E] int64 from sigmoid_q23, bias
+    [E] int32 or None -> (weights [T,topk] int64, indices [T,topk] int64).  `raw_weights`, if given, receives the
+    winners' unbiased scores (what the reference dumps as gate_weights.bin)."""
+    assert scores.is_cuda and scores.dtype == torch.int64 and scores.is_contiguous() and scores.dim() == 2
+    assert bias is None or (bias.is_cuda and bias.dtype == torch.int32 and bias.is_contiguous() and bias.numel() == scores.shape[1])
+    T, E = scores.shape
+    weights = torch.empty((T, topk), dtype=torch.int64, device=scores.device)
+    indices = torch.empty((T, topk), dtype=torch.int64, device=scores.device)
+    lib.gate_route_q23(scores.data_ptr(), 0 if bias is None else bias.data_ptr(), weights.data_ptr(), indices.data_ptr(),
+                       0 if raw_weights is None else raw_weights.data_ptr(), T, E, n_groups, topk_groups, topk)
+    _check("gate_route_q23")
+    return weights, indices
 
 
 def silu_mul_q23(R, U, C, S=None):
