@@ -251,6 +251,38 @@ def main():
             hbm("gate_route_%dx256" % Tt, lambda: K.gate_route(gsc, gbias, 8, 4, 8), Tt, bytes_per_elem=8.0 * 256 + 128.0, steps=20)
             del gsc
 
+        # witness dump: what one layer's ~30 saveTensor calls cost the host thread, against the reference's way
+        # (synchronous .cpu() + tobytes + write, inference/model.py:94-102); files go to a temporary directory
+        import shutil
+        import tempfile
+        tmpd = tempfile.mkdtemp(prefix="zkdump_")
+        try:
+            dumps = [randint(gr, -(1 << 40), 1 << 40, (256, 7168)).cuda() for _ in range(30)]
+            torch.cuda.synchronize()
+
+            def ref_style():
+                for i, t in enumerate(dumps):
+                    with open(os.path.join(tmpd, "r%d.bin" % i), "wb") as f:
+                        f.write(t.cpu().contiguous().numpy().tobytes(order="C"))
+
+            ref_style()
+            t0 = time.perf_counter()
+            ref_style()
+            ref_ms = (time.perf_counter() - t0) * 1e3
+            for rep in range(2):
+                t0 = time.perf_counter()
+                for i, t in enumerate(dumps):
+                    K.saveTensor(os.path.join(tmpd, "a%d.bin" % i), t)
+                queued_ms = (time.perf_counter() - t0) * 1e3
+                K.dump_flush()
+                total_ms = (time.perf_counter() - t0) * 1e3
+            nbytes = sum(t.numel() * 8 for t in dumps)
+            extra["witness_dump_30x256x7168"] = {"bytes": nbytes, "host_blocked_ms": queued_ms, "until_flushed_ms": total_ms,
+                                                 "reference_style_ms": ref_ms}
+            del dumps
+        finally:
+            shutil.rmtree(tmpd, ignore_errors=True)
+
         # RoPE and the float -> fixed converters (weight-loading path), by their own algorithmic bytes per element
         gq = torch.Generator(device="cpu").manual_seed(700)
         q_pe = randint(gq, -(1 << 30), 1 << 30, (1, 4096, 128, 32, 2)).cuda()

@@ -19,6 +19,7 @@
 #ifndef ZK_INT64GEMM_H
 #define ZK_INT64GEMM_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -137,6 +138,17 @@ void silu_mul_q23(const int64_t *R, const int64_t *U, int64_t *S, int64_t *C, co
  * weights [T,topk] = floor(floor(raw * 2^23 / sum raw) * 5 / 2).  E <= 1024, n_groups <= 64 dividing E, topk <= 64. */
 void gate_route_q23(const int64_t *scores, const int32_t *bias, int64_t *weights, int64_t *indices,
                     int64_t *raw_weights, int T, int E, int n_groups, int topk_groups, int topk);
+
+/* Witness dump writer (replaces the reference's saveTensor, inference/model.py:94-102: a synchronous .cpu() copy and
+ * file write per tensor, ~30 per layer).  zk_dump_device queues the raw bytes of `bytes` bytes of contiguous device
+ * memory for `path`: the copy to pinned host memory is ordered on the null stream behind the kernels that produced
+ * the data and ahead of anything launched later, so the caller may overwrite or free the tensor right after the call
+ * returns; a writer thread writes the file (created or truncated) once the copy has landed.  zk_dump_host does the
+ * same for host memory (copied before it returns).  Both return 0, or -1 with zk_last_error set.  Files are complete
+ * only after zk_dump_flush(), which waits for everything queued and returns the number of dumps that failed. */
+int zk_dump_device(const char *path, const void *device_ptr, size_t bytes);
+int zk_dump_host(const char *path, const void *host_ptr, size_t bytes);
+long zk_dump_flush(void);
 
 /* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */

@@ -78,3 +78,33 @@ def test_kernel_module_mirrors_reference_api():
     assert kernel.rms.shape == (500,) and kernel.rms.device.type == "cpu"
     with pytest.raises(NotImplementedError):
         kernel.fp8_gemm()
+
+
+def test_dump_writer_host_path(lib, tmp_path):
+    """the witness dump writer on host memory (no GPU needed): bytes identical to numpy's tobytes, large tensors go
+    through in pieces, an unwritable path is reported by the flush"""
+    lib.zk_dump_host.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t]
+    lib.zk_dump_flush.restype = ctypes.c_long
+    lib.zk_last_error_string.restype = ctypes.c_char_p
+    lib.zk_clear_error()
+    rng = np.random.default_rng(1)
+    arrays = {"empty.bin": np.zeros(0, np.int64), "one.bin": np.array([-5], np.int64),
+              "w32.bin": rng.integers(-(1 << 31), 1 << 31, size=(37, 129), dtype=np.int64).astype(np.int32),
+              "big.bin": rng.integers(-(1 << 62), 1 << 62, size=(5 << 20) + 3, dtype=np.int64)}       # 40 MB: two pieces
+    for name, a in arrays.items():
+        assert lib.zk_dump_host(os.fsencode(str(tmp_path / name)), ctypes.c_void_p(a.ctypes.data), a.nbytes) == 0
+    big = arrays["big.bin"]
+    big[:] = 0                                             # the data was copied before the call returned
+    assert lib.zk_dump_flush() == 0
+    rng = np.random.default_rng(1)
+    want = {"empty.bin": np.zeros(0, np.int64), "one.bin": np.array([-5], np.int64),
+            "w32.bin": rng.integers(-(1 << 31), 1 << 31, size=(37, 129), dtype=np.int64).astype(np.int32),
+            "big.bin": rng.integers(-(1 << 62), 1 << 62, size=(5 << 20) + 3, dtype=np.int64)}
+    for name, a in want.items():
+        assert (tmp_path / name).read_bytes() == a.tobytes(order="C"), name
+    a = np.arange(4, dtype=np.int64)
+    assert lib.zk_dump_host(os.fsencode(str(tmp_path / "no_such_dir" / "x.bin")), ctypes.c_void_p(a.ctypes.data), a.nbytes) == 0
+    assert lib.zk_dump_flush() == 1
+    assert b"no_such_dir" in lib.zk_last_error_string()
+    lib.zk_clear_error()
+    assert lib.zk_dump_flush() == 0

@@ -570,6 +570,38 @@ def test_gate_route(K, oracle, E, G, KG, K_, with_bias):
         assert np.array_equal(host(w), we), "weights"
 
 
+def test_witness_dump_writer(K, tmp_path):
+    """saveTensor through the library's writer: same bytes as the reference's t.cpu().numpy().tobytes(), for device and
+    host tensors, views, large tensors (several staging pieces) and many small files; a tensor overwritten right
+    after the call still lands in the file with the contents it had at the call"""
+    g = torch.Generator(device="cpu").manual_seed(9)
+    cases = {
+        "scores.bin": torch.randint(-(1 << 62), 1 << 62, (3, 5, 7, 11), generator=g).cuda(),
+        "weights_u32.bin": torch.randint(-(1 << 31), 1 << 31, (129, 37), generator=g).to(torch.int32).cuda().view(torch.int32),
+        "strided.bin": torch.randint(-9, 9, (64, 48), generator=g).cuda()[:, ::3],
+        "host.bin": torch.randint(-9, 9, (1000,), generator=g),
+        "big.bin": torch.randint(-(1 << 62), 1 << 62, ((13 << 20) + 5,), generator=g).cuda(),          # 104 MB: four pieces
+    }
+    want = {k: v.detach().cpu().contiguous().numpy().tobytes(order="C") for k, v in cases.items()}
+    for name, t in cases.items():
+        K.saveTensor(str(tmp_path / name), t)
+    cases["big.bin"].zero_()                                   # queued behind the copy
+    cases["scores.bin"].fill_(7)
+    small = [torch.full((17,), i, dtype=torch.int64, device="cuda") for i in range(100)]
+    for i, t in enumerate(small):
+        K.saveTensor(str(tmp_path / ("small_%d.bin" % i)), t)
+        t.add_(1000)
+    K.dump_flush()
+    for name, b in want.items():
+        assert (tmp_path / name).read_bytes() == b, name
+    for i in range(100):
+        assert (tmp_path / ("small_%d.bin" % i)).read_bytes() == np.full(17, i, np.int64).tobytes()
+    K.saveTensor(str(tmp_path / "missing_dir" / "x.bin"), small[0])
+    with pytest.raises(RuntimeError):
+        K.dump_flush()
+    K.lib.zk_clear_error()
+
+
 def test_converters(K, oracle):
     """the three float -> fixed converters the reference exports (inference/int64_gemm.cu:92-221)"""
     rng = np.random.default_rng(31)

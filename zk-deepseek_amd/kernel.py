@@ -14,6 +14,7 @@ Differences from the reference, all deliberate:
     importable names that raise NotImplementedError.
 There is no CPU fallback: if the shared object is missing, importing this module raises.
 """
+import atexit
 import ctypes
 import os
 
@@ -68,6 +69,9 @@ lib.zk_gemm_guard_hits.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
 lib.gate_route_q23.argtypes = [_vp] * 5 + [_ci] * 5
+lib.zk_dump_device.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
+lib.zk_dump_host.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
+lib.zk_dump_flush.restype = ctypes.c_long
 lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
 
@@ -220,6 +224,9 @@ def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim):
     return (C, rms)
 
 
+atexit.register(lambda: lib.zk_dump_flush())
+
+
 def saveTensor(fileName, t):
     """Raw C-order little-endian bytes, the witness format the proving side reads back."""
     t = t.detach()
@@ -317,6 +324,28 @@ def softmax_q19_scores(s1, s2, mask, C, scores=None, mul=94, div=695):
     lib.softmax_q19_scores(s1.data_ptr(), ptr(s2), ptr(mask), ptr(scores), C.data_ptr(), EXP2_FRAC_LUT_Q19.data_ptr(),
                            Bsz, S, H, T, int(mul), int(div))
     _check("softmax_q19_scores")
+
+
+def saveTensor(fileName, t):
+    """The reference's saveTensor (inference/model.py:94-102) without the wait: the raw C-order bytes of `t` go to
+    `fileName` through the library's dump writer.  Device tensors are copied behind the work already queued on the GPU,
+    so `t` may be overwritten or freed right after this returns; host tensors are copied before it returns.  Call
+    `dump_flush()` before reading the files (it also runs at interpreter exit)."""
+    t = t.detach()
+    if not t.is_contiguous():
+        t = t.contiguous()
+    nbytes = t.numel() * t.element_size()
+    fn = lib.zk_dump_device if t.is_cuda else lib.zk_dump_host
+    if fn(os.fsencode(fileName), t.data_ptr(), nbytes) != 0:
+        _check("saveTensor")
+    # a temporary made contiguous above stays alive until the copy is queued: device copies are stream ordered and
+    # torch's allocator only hands the memory to work queued later; host data has been copied already
+
+
+def dump_flush():
+    """wait until every tensor passed to saveTensor is in its file; raises if any write failed"""
+    if lib.zk_dump_flush() != 0:
+        _check("dump_flush")
 
 
 def gate_route(scores, bias, n_groups, topk_groups, topk, raw_weights=None):
