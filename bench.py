@@ -251,6 +251,26 @@ def main():
             hbm("gate_route_%dx256" % Tt, lambda: K.gate_route(gsc, gbias, 8, 4, 8), Tt, bytes_per_elem=8.0 * 256 + 128.0, steps=20)
             del gsc
 
+        # config 5's routed experts: 256 tokens, top 8 of 256 experts of width 2048 on dim 7168, int64 weights resident
+        # (90.2 GB): bound by the one pass over the weights.  Routing, dispatch, three grouped GEMM launches, combine.
+        free_b, _tot = torch.cuda.mem_get_info()
+        if free_b > 110 * (1 << 30):
+            gm = torch.Generator(device="cuda").manual_seed(5001)
+            mkw = lambda *shape: torch.randint(-(1 << 16), 1 << 16, shape, generator=gm, dtype=torch.int64, device="cuda")
+            ew1 = [mkw(2048, 7168) for _ in range(256)]
+            ew3 = [mkw(2048, 7168) for _ in range(256)]
+            ew2 = [mkw(7168, 2048) for _ in range(256)]
+            tabs = [K.pointer_table(w) for w in (ew1, ew3, ew2)]
+            xm = randint(gr, -(1 << 20), 1 << 20, (256, 7168)).cuda()
+            sm = randint(gr, 1, 1 << 23, (256, 256)).cuda()
+            wm, im = K.gate_route(sm, gbias, 8, 4, 8)
+            wbytes = 3.0 * 256 * 2048 * 7168 * 8
+            hbm("moe_experts_config5_256tok_top8_of_256", lambda: K.moe_experts(xm, wm, im, tabs[0], tabs[1], tabs[2], False, 2048, 17, 20),
+                1, bytes_per_elem=wbytes, steps=3)
+            extra["moe_experts_config5_256tok_top8_of_256"]["weight_bytes"] = wbytes
+            del ew1, ew3, ew2, tabs
+            torch.cuda.empty_cache()
+
         # witness dump: what one layer's ~30 saveTensor calls cost the host thread, against the reference's way
         # (synchronous .cpu() + tobytes + write, inference/model.py:94-102); files go to a temporary directory
         import shutil

@@ -150,6 +150,30 @@ int zk_dump_device(const char *path, const void *device_ptr, size_t bytes);
 int zk_dump_host(const char *path, const void *host_ptr, size_t bytes);
 long zk_dump_flush(void);
 
+/* MoE dispatch on the device (no counterpart in the reference's library; together these replace the Python loop over
+ * the experts of MoE.forward, inference/model.py:1325-1383).  All pointers are device pointers.
+ *
+ * moe_dispatch: indices [T,K] int64 (expert of every routed (token, slot) entry, as gate_route_q23 returns them) ->
+ *   seg [E+1]: first row of every expert's segment in the sorted order (seg[E] = T*K);
+ *   sorted_token [T*K]: the token of every sorted row (tokens ascending within an expert, as torch.where gives them);
+ *   sorted_pos [T*K]: the sorted row of entry (t, k);
+ *   tiles [2 * (T*K/32 + E)], ntiles [1]: the 32-row tiles of the segments, for int64_grouped_bmm_launcher;
+ *   counts_scratch [E]: scratch.
+ * moe_gather_rows: out[r][:] = x[sorted_token[r]][:]  (x [T,N], out [rows,N]).
+ * int64_grouped_bmm_launcher: C[r][n] = (sum_k A[r][k] * B_e[n][k]) >> c_rescale (128-bit wrapping sum) and, when R
+ *   is not null, R = that sum mod 2^c_rescale, for the rows r of expert e's segment; B_ptrs [groups] holds the
+ *   experts' weight matrices ([N,K], int32 when b32 else int64).  Semantics of int64_64/32_bmm_broadcast_launcher
+ *   per segment.  It waits for the device once per call (its digit check; see zk_gemm_guard_hits).
+ * moe_combine: y[t][n] = sum_k (ye[sorted_pos[t][k]][n] * weights[t][k]) >> shift with wrapping products and sums
+ *   (model.py:1379 with shift 23; floor, like torch's //). */
+void moe_dispatch(const int64_t *indices, int T, int K, int E, int *counts_scratch, int *seg, int *sorted_token,
+                  int *sorted_pos, int *tiles, int *ntiles);
+void moe_gather_rows(const int64_t *x, const int *sorted_token, int64_t *out, int rows, int N);
+void int64_grouped_bmm_launcher(const int64_t *A, const void *const *B_ptrs, int b32, int64_t *C, int64_t *R,
+                                int64_t c_rescale, const int *seg, const int *tiles, const int *ntiles, int groups,
+                                int rows, int K, int N);
+void moe_combine(const int64_t *ye, const int64_t *weights, const int *sorted_pos, int64_t *y, int T, int K, int N, int shift);
+
 /* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
 void zk_gemm_set_path(int path);
@@ -161,6 +185,8 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
  * behind it recomputes the outputs if the guess was too small.  This returns how many calls so far needed that
  * recomputation (counted once their ranges have reached the host; it waits for nothing). */
 long zk_gemm_guard_hits(void);
+/* How many int64_grouped_bmm_launcher calls so far ran as ONE launch over all groups (the others went group by group). */
+long zk_gemm_grouped_mfma_calls(void);
 
 /* Measurement helper for the roofline of the MFMA GEMM path: the sustained rate, in 10^12 i8 operations per
  * second (2 per multiply-add), of a stream of v_mfma_i32_32x32x32_i8 shaped like the GEMM's inner loop (8 waves

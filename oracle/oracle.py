@@ -267,6 +267,51 @@ def gate_route(scores, bias, n_groups, topk_groups, topk):
     return w, idx, raw
 
 
+def moe_dispatch(indices, n_experts):
+    """(seg [E+1], sorted_token [T*K], sorted_pos [T,K]): the (token, slot) entries sorted by expert, stably, so an
+    expert sees its tokens in ascending order (what torch.where gives MoE.forward, inference/model.py:1357-1365)"""
+    T, K = indices.shape
+    flat = np.asarray(indices).ravel()
+    order = np.argsort(flat, kind="stable")
+    seg = np.concatenate([[0], np.cumsum(np.bincount(flat, minlength=n_experts))]).astype(np.int32)
+    pos = np.empty(T * K, np.int32)
+    pos[order] = np.arange(T * K, dtype=np.int32)
+    return seg, (order // K).astype(np.int32), pos.reshape(T, K)
+
+
+def grouped_bmm(A_sorted, weights_list, seg, c_rescale):
+    """(C, R) [rows,N]: int64_bmm_broadcast of every expert's segment of rows with that expert's matrix"""
+    N = weights_list[0].shape[0]
+    C = np.zeros((A_sorted.shape[0], N), np.int64)
+    R = np.zeros_like(C)
+    for e, w in enumerate(weights_list):
+        r0, r1 = int(seg[e]), int(seg[e + 1])
+        if r1 > r0:
+            c, r = int64_bmm_broadcast(np.ascontiguousarray(A_sorted[None, r0:r1]), w, 1, 1, c_rescale)
+            C[r0:r1], R[r0:r1] = c[0], r[0]
+    return C, R
+
+
+def moe_experts(x, weights, indices, w1, w3, w2, c13, c2):
+    """The routed experts of MoE.forward as the reference loops over them (inference/model.py:1355-1381): for every
+    expert with tokens, Expert_int.forward on those tokens (:1247-1281), times the routing weight, floor-divided by
+    2^23 and added to the tokens' rows."""
+    T, dim = x.shape
+    y = np.zeros((T, dim), np.int64)
+    for e in range(len(w1)):
+        tok, slot = np.nonzero(np.asarray(indices) == e)
+        if tok.size == 0:
+            continue
+        xe = np.ascontiguousarray(x[tok])[None]
+        r1, _ = int64_bmm_broadcast(xe, w1[e], 1, 1, c13)
+        r2, _ = int64_bmm_broadcast(xe, w3[e], 1, 1, c13)
+        _, h = silu_mul_q23(r1, r2)
+        ye, _ = int64_bmm_broadcast(h, w2[e], 1, 1, c2)
+        with np.errstate(over="ignore"):
+            np.add.at(y, tok, (ye[0] * weights[tok, slot][:, None]) >> 23)
+    return y
+
+
 def bf16_to_int32_2d(bits, rescale):
     """bits: uint16 bf16 patterns [rows, cols] -> int32 fixed point (inference/int64_gemm.cu:92-132)"""
     bits = _c(bits, np.uint16)

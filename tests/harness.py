@@ -138,7 +138,19 @@ class FusedGpuBackend(GpuBackend):
     def route(self, scores, bias_host, cfg):
         bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
         w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"])
+        self.last_route = (w, idx)
         return w.cpu().numpy(), idx.cpu().numpy()
+
+    def routed_experts(self, x, P, cfg):
+        """every routed expert in one go, from the routing result that is still on the device"""
+        w, idx = self.last_route
+        key = id(P["w1"])
+        if getattr(self, "_tables_for", None) != key:
+            self._tables = tuple(self.k.pointer_table(P[n]) for n in ("w1", "w3", "w2"))
+            self._tables_for = key
+        t1, t3, t2 = self._tables
+        b32 = P["w1"][0].dtype == self.t.int32
+        return self.k.moe_experts(x[0].contiguous(), w, idx, t1, t3, t2, b32, cfg["inter"], cfg["c13"], cfg["c2"])
 
 
 class CheckedGpuBackend(GpuBackend):
@@ -300,6 +312,10 @@ def moe(be, x, P, cfg):
     T = x.shape[1]
     sc = gate_scores(be, x, P, cfg)
     w_host, idx_host = be.route(sc, P["gate_bias_host"], cfg) if hasattr(be, "route") else route(be.to_host(sc), P["gate_bias_host"], cfg)
+    if hasattr(be, "routed_experts"):
+        y = be.routed_experts(x, P, cfg)
+        z = expert_ffn(be, x, P["sw1"], P["sw2"], P["sw3"], cfg["c13"], cfg["c2"])
+        return y[None] + z, idx_host
     y = be.zeros_like(x[0])
     for e in range(cfg["experts"]):
         tok, slot = np.nonzero(idx_host == e)

@@ -168,6 +168,12 @@ def test_config5_decoder_layer_full_size(backends):
     assert c["linear"] > 3 * 48 * (6 + 3 * 200) and c["softmax"] >= 4096 * S and c["rmsnorm"] == S * (2 * dim + 1536 + 512)
     for name in ("einsum_bshd_hdc_bshc", "einsum_bshc_btc_bsht", "einsum_bsht_btc_bshc", "einsum_bshc_hdc_bshd", "silu", "sigmoid", "rope"):
         assert c.get(name, 0) > 0, name
+    # the same layer through the fused entry points and the device-side MoE (routing, dispatch, ONE grouped launch per
+    # expert matrix over all 256 experts, combine): identical output
+    before = kernel.lib.zk_gemm_grouped_mfma_calls()
+    y2, idx2 = H.decoder_layer(H.FusedGpuBackend(kernel), x, P, freqs, cfg)
+    assert kernel.lib.zk_gemm_grouped_mfma_calls() - before == 3
+    assert np.array_equal(idx2, idx) and torch.equal(y2, y)
     # the layer's output is alive: neither stuck at the residual nor saturated
     d = (y - x).abs()
     assert int(d.max()) > 0 and int(y.abs().max()) < 1 << 62

@@ -570,6 +570,75 @@ def test_gate_route(K, oracle, E, G, KG, K_, with_bias):
         assert np.array_equal(host(w), we), "weights"
 
 
+def _routing(rng, T, E, Kr):
+    """Kr distinct experts per token; some experts deliberately left without tokens"""
+    live = rng.permutation(E)[: max(Kr, (E * 3) // 4)]
+    return np.stack([rng.permutation(live)[:Kr] for _ in range(T)]).astype(np.int64)
+
+
+@pytest.mark.parametrize("T,E,Kr", [(1, 8, 2), (5, 4, 4), (100, 16, 3), (256, 256, 8), (700, 32, 6)])
+def test_moe_dispatch(K, oracle, T, E, Kr):
+    rng = np.random.default_rng(T + E)
+    idx = _routing(rng, T, E, Kr)
+    d = K.moe_dispatch(dev(idx), E)
+    seg, tok, pos = oracle.moe_dispatch(idx, E)
+    assert np.array_equal(host(d["seg"]), seg)
+    assert np.array_equal(host(d["token"]), tok)
+    assert np.array_equal(host(d["pos"]), pos)
+    nt = int(host(d["ntiles"])[0])
+    tiles = host(d["tiles"])[: 2 * nt].reshape(nt, 2)
+    want = [(e, r) for e in range(E) for r in range(int(seg[e]), int(seg[e + 1]), 32)]
+    assert tiles.tolist() == [list(t) for t in want]
+
+
+@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("w32", [False, True])
+@pytest.mark.parametrize("bits", [(20, 16), (37, 30), (50, 31)])
+def test_int64_grouped_bmm(K, oracle, path, w32, bits):
+    """one launch over all experts against the per-expert oracle GEMMs: empty experts, experts with more than 32
+    rows, ragged K and N, the remainder output; (50, 31)-bit operands are wider than the 32-row kernels take and go
+    expert by expert"""
+    rng = np.random.default_rng(bits[0] + w32)
+    T, E, Kr, Kd, N = 90, 12, 3, 200, 300
+    idx = _routing(rng, T, E, Kr)
+    idx[:60, 0] = 2                                           # expert 2 gets more than 32 rows
+    idx[:60, 1:] = np.stack([rng.permutation([0, 1, 3, 4, 5])[: Kr - 1] for _ in range(60)])
+    x = rand_i64(rng, (T, Kd), bits[0])
+    ws = [rand_i32(rng, (N, Kd), bits[1]) if w32 else rand_i64(rng, (N, Kd), bits[1]) for _ in range(E)]
+    K.lib.zk_gemm_set_path(path)
+    d = K.moe_dispatch(dev(idx), E)
+    xs = K.moe_gather_rows(dev(x), d)
+    seg, tok, _ = oracle.moe_dispatch(idx, E)
+    assert np.array_equal(host(xs), x[tok])
+    wd = [dev(w) for w in ws]
+    before = K.lib.zk_gemm_grouped_mfma_calls()
+    for c in (0, 19):
+        C, R = K.int64_grouped_bmm(xs, K.pointer_table(wd), w32, N, c, d, want_remainder=True)
+        Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
+        assert np.array_equal(host(C), Ce), "quotient"
+        assert np.array_equal(host(R), Re), "remainder"
+    single_launch = path != 1 and bits[0] <= 39
+    assert K.lib.zk_gemm_grouped_mfma_calls() - before == (2 if single_launch else 0), "which route the product took"
+    K.lib.zk_gemm_set_path(0)
+
+
+@pytest.mark.parametrize("w32", [False, True])
+def test_moe_experts(K, oracle, w32):
+    """routed experts end to end (dispatch, gather, grouped gate/up GEMMs, SiLU gate, grouped down GEMM, weighted
+    combine) against the reference's loop over the experts restated on the oracle"""
+    rng = np.random.default_rng(11 + w32)
+    T, E, Kr, dim, inter = 40, 8, 3, 96, 160
+    idx = _routing(rng, T, E, Kr)
+    x = rand_i64(rng, (T, dim), 24)
+    wts = rng.integers(1, 1 << 23, size=(T, Kr), dtype=np.int64)
+    mk = (lambda shape: rand_i32(rng, shape, 27)) if w32 else (lambda shape: rand_i64(rng, shape, 27))
+    w1, w3, w2 = [mk((inter, dim)) for _ in range(E)], [mk((inter, dim)) for _ in range(E)], [mk((dim, inter)) for _ in range(E)]
+    d1, d3, d2 = [dev(w) for w in w1], [dev(w) for w in w3], [dev(w) for w in w2]
+    y = K.moe_experts(dev(x), dev(wts), dev(idx), K.pointer_table(d1), K.pointer_table(d3), K.pointer_table(d2), w32, inter, 29, 27)
+    ye = oracle.moe_experts(x, wts, idx, w1, w3, w2, 29, 27)
+    assert np.array_equal(host(y), ye)
+
+
 def test_witness_dump_writer(K, tmp_path):
     """saveTensor through the library's writer: same bytes as the reference's t.cpu().numpy().tobytes(), for device and
     host tensors, views, large tensors (several staging pieces) and many small files; a tensor overwritten right

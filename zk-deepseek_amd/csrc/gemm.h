@@ -38,6 +38,33 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 // vector-ALU recomputation (known once their range has reached the host).
 long gemm_mfma_guard_hits();
 
+// Grouped product: the rows of A and C form one contiguous segment per group and every group has its own
+// k-contiguous B[N,K] (the experts of a MoE layer after the tokens have been sorted by expert):
+//   C[r][n] = (init + sum_k A[r][k] * B_group(r)[n][k]) >> shift,   R likewise.
+// Everything that describes the segments lives on the device, so the host never learns the segment sizes.
+struct GroupedDesc {
+    const int64_t *A;
+    long lda;
+    const void *const *B;     // device array of `groups` device pointers
+    int b32;
+    int64_t *C, *R;           // R may be null
+    long ldc;
+    const int *seg;           // device [groups + 1]: first row of every segment, seg[groups] = rows
+    const int *tiles;         // device [2 * (rows / 32 + groups)]: {group, first row} of every 32-row tile
+    const int *ntiles;        // device [1]: how many of those tiles exist
+    int groups, rows, N, K, shift;
+    int64_t init;
+};
+
+// One launch of the 32-row-tile MFMA kernels over all groups.  Returns 0 when done, 1 when the operands need
+// more digits than those kernels are built for (nothing valid was written: the caller takes another route),
+// -1 on an error (recorded).
+int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b);
+
+// Grouped product through the MFMA launch above or, where that does not apply (path forced to VALU, K = 0,
+// operands wider than its kernels take), group by group through gemm_dispatch after one read-back of the segments.
+void gemm_grouped_dispatch(const char *name, const GroupedDesc &d);
+
 // Top-level dispatch used by the extern "C" launchers.
 void gemm_dispatch(const char *name, const GemmDesc &d);
 

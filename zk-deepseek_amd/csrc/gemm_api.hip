@@ -3,10 +3,13 @@
 #include "gemm.h"
 #include "../../include/int64gemm.h"
 
+#include <vector>
+
 namespace zk {
 
 static int g_gemm_path = kPathAuto;
 static int g_last_path = 0, g_last_la = 0, g_last_lb = 0;
+static long g_grouped_mfma_calls = 0;
 
 void gemm_dispatch(const char *name, const GemmDesc &d)
 {
@@ -22,6 +25,41 @@ void gemm_dispatch(const char *name, const GemmDesc &d)
     gemm_valu_launch(d);
     g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
     check_launch(name);
+}
+
+void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
+{
+    if (g_gemm_path != kPathValu && d.K > 0) {
+        int la = 0, lb = 0;
+        const int rc = gemm_mfma_grouped(d, &la, &lb);
+        if (rc == 0) {
+            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb;
+            g_grouped_mfma_calls++;
+            check_launch(name);
+            return;
+        }
+        if (rc < 0) return;
+    }
+    // group by group: the segment table and the B pointers come to the host once
+    std::vector<int> seg((size_t)d.groups + 1);
+    std::vector<const void *> bp((size_t)d.groups);
+    if (hipMemcpy(seg.data(), d.seg, seg.size() * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy(bp.data(), d.B, bp.size() * sizeof(void *), hipMemcpyDeviceToHost) != hipSuccess) {
+        set_error(kLaunchFailure, "%s: cannot read the segment table", name);
+        return;
+    }
+    for (int e = 0; e < d.groups; e++) {
+        const int r0 = seg[e], m = seg[e + 1] - seg[e];
+        if (m <= 0) continue;
+        GemmDesc g;
+        g.A = d.A + (long)r0 * d.lda; g.lda = d.lda; g.sA = 0;
+        g.B = bp[e]; g.b32 = d.b32; g.ldbn = d.K; g.ldbk = 1; g.sB = 0;
+        g.C = d.C + (long)r0 * d.ldc; g.R = d.R ? d.R + (long)r0 * d.ldc : nullptr; g.ldc = d.ldc; g.sC = 0;
+        g.G = 1; g.M = m; g.N = d.N; g.K = d.K;
+        g.shift = d.shift; g.init = d.init; g.a_rs = 1; g.b_rs = 1;
+        gemm_dispatch(name, g);
+        if (zk_last_error() != kOk) return;
+    }
 }
 
 static bool dims_ok(const char *name, std::initializer_list<int> dims, int64_t shift)
@@ -153,5 +191,7 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b)
 }
 
 long zk_gemm_guard_hits(void) { return zk::gemm_mfma_guard_hits(); }
+
+long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
 
 }  // extern "C"

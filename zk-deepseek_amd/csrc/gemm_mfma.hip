@@ -65,6 +65,12 @@ struct MfmaParams {
     int main_tiles, split;
     unsigned long long *partials;
     int part64;                     // the partial sums fit 64 bits: only the low words are kept
+    // grouped mode (GRP kernels): rows of A and C form one segment per group, each group has its own B.
+    // Workgroup (mt, tn) looks up 32-row tile mt in grp_tiles = {group, first row} and stops at the segment's end.
+    const int *grp_seg;             // [groups + 1] first row of every segment
+    const int *grp_tiles;           // [2 * tiles] group and first row of every 32-row tile
+    const int *grp_ntiles;          // how many of them exist (the grid is sized for the worst case)
+    const void *const *grp_b;       // [groups] B of every group
     int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
 };
 
@@ -366,7 +372,7 @@ __global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long lon
 // outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
 // own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
 // to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
-template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL>
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 {
     constexpr int T = 64 * WVM * WVN;
@@ -386,19 +392,40 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     // fastest, so the workgroups that share a B tile sit on the same L2.
     const int per_batch = p.tiles_m * p.tiles_n;
     int lin = blockIdx.x, sidx = 0, nsplit = 1;
-    if (lin < p.main_tiles) {
-        if ((p.main_tiles & 7) == 0) lin = (lin & 7) * (p.main_tiles >> 3) + (lin >> 3);
+    int tail_tile = 0, g = 0, tn, tm, m0, m_lim = p.M;
+    const void *b_base = p.B;
+    if (GRP) {
+        const int mt = lin / p.tiles_n;
+        if (mt >= *p.grp_ntiles) {                 // the grid covers the worst case: nothing to do, an empty range
+            if (tid == 0) {
+                unsigned long long *slot = p.wg_range + 4 * (long)blockIdx.x;
+                slot[0] = ~0ull; slot[1] = 0ull; slot[2] = ~0ull; slot[3] = 0ull;
+            }
+            return;
+        }
+        tn = lin - mt * p.tiles_n;
+        tm = 0;
+        const int e = p.grp_tiles[2 * mt];
+        m0 = p.grp_tiles[2 * mt + 1];
+        m_lim = p.grp_seg[e + 1];
+        b_base = p.grp_b[e];
     } else {
-        const int t = lin - p.main_tiles;
-        lin = p.main_tiles + t / p.split;
-        sidx = t % p.split;
-        nsplit = p.split;
+        if (lin < p.main_tiles) {
+            if ((p.main_tiles & 7) == 0) lin = (lin & 7) * (p.main_tiles >> 3) + (lin >> 3);
+        } else {
+            const int t = lin - p.main_tiles;
+            lin = p.main_tiles + t / p.split;
+            sidx = t % p.split;
+            nsplit = p.split;
+        }
+        tail_tile = lin - p.main_tiles;            // index among the split tiles (when nsplit > 1)
+        g = lin / per_batch;
+        const int rem = lin - g * per_batch;
+        tn = rem / p.tiles_m;
+        tm = rem - tn * p.tiles_m;
+        m0 = tm * BM;
     }
-    const int tail_tile = lin - p.main_tiles;      // index among the split tiles (when nsplit > 1)
-    const int g = lin / per_batch;
-    const int rem = lin - g * per_batch;
-    const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int n0 = tn * BN;
 
     // Range tracking is shared out: the tiles_m workgroups that load the same B tile each check every
     // tiles_m-th k-step of it (likewise for A across the workgroups of a tile row), so no workgroup is slower
@@ -426,7 +453,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     v4i pa[A_CIT];
 
     const bool a_vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
-    const bool b_vec = !BKM && (((uintptr_t)p.B | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
+    const bool b_vec = !BKM && (((uintptr_t)b_base | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
 
     // per-thread source pointers (advanced by BK per step) and LDS destinations
     const int64_t *a_src[A_IT];
@@ -458,7 +485,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             const int row = (live ? idx : 0) / OCTS;
             a_j[it] = idx % OCTS;
             int m = m0 + row;
-            m = m < p.M ? m : p.M - 1;
+            m = m < m_lim ? m : m_lim - 1;
             a_src[it] = p.A + (long)g * p.sA + (long)m * p.lda;
             a_dst[it] = live ? frag_offset(row, a_j[it], NA, SUBSTAGE) : DUMMY;
             a_stride[it] = live ? STAGE : 0;
@@ -475,7 +502,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         int n = n0 + row;
         n = n < p.N ? n : p.N - 1;
         const long off = (long)g * p.sB + (long)n * p.ldbn;
-        b_src[it] = reinterpret_cast<const char *>(p.B) + off * (B32 ? 4 : 8);
+        b_src[it] = reinterpret_cast<const char *>(b_base) + off * (B32 ? 4 : 8);
         b_dst[it] = live ? A_BLOCKS * 1024 + frag_offset(row, b_j[it], NB, SUBSTAGE) : DUMMY;
         b_stride[it] = live ? STAGE : 0;
     }
@@ -687,7 +714,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             for (int r = 0; r < 16; r++) {
                 const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 // rows of this register that all lie past M (uniform over the wave): nothing to keep
-                if (nsplit > 1 && m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= p.M) continue;
+                if (nsplit > 1 && m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= m_lim) continue;
                 // whole tiles start from the rounding term; split workgroups leave it to the finishing kernel
                 uint64_t lo = nsplit > 1 ? 0 : (uint64_t)p.init, hi = nsplit > 1 ? 0 : (uint64_t)(p.init >> 63);
 #pragma unroll
@@ -708,7 +735,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                     const long q = (((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r;
                     if (p.part64) p.partials[q * 64 + lane] = lo;
                     else { p.partials[q * 128 + lane] = lo; p.partials[q * 128 + 64 + lane] = hi; }
-                } else if (m < p.M && n < p.N) {
+                } else if (m < m_lim && n < p.N) {
                     const long o = (long)g * p.sC + (long)m * p.ldc + n;
                     uint64_t q;
                     if (p.shift == 0) q = lo;
@@ -778,7 +805,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
 typedef void (*MfmaKernel)(MfmaParams);
 typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
 
-enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kVariants };
+enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kVariants };
 
 struct Instance {
     int na, nb, bm, bn, threads, kk;
@@ -812,6 +839,10 @@ static Instance make_instance()
         s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false>;
         s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true>;
         s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false>;
+    }
+    if constexpr (SKINNY) {          // grouped launches (one B per segment of rows) run on the 32-row tiles only
+        s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true>;
+        if constexpr (NB <= 5) s.fn[kB32Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, true>;
     }
     s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
     s.planes[0] = a_planes_kernel<NA, 2, KK>;
@@ -1138,6 +1169,79 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     }
     set_error(kLaunchFailure, "gemm: digit count did not settle");
     return false;
+}
+
+int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
+{
+    if (d.K <= 0 || d.N <= 0 || d.rows <= 0 || d.groups <= 0) return 1;
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    if (!init_cache()) return -1;
+    drain_pending();
+
+    MfmaParams p = {};
+    p.A = d.A; p.B = nullptr; p.C = d.C; p.R = d.R;
+    p.lda = d.lda; p.sA = 0; p.ldbn = d.K; p.ldbk = 1; p.sB = 0; p.ldc = d.ldc; p.sC = 0;
+    p.M = d.rows; p.N = d.N; p.K = d.K; p.shift = d.shift; p.init = d.init;
+    p.range = g_cache.dev;
+    p.tiles_m = 1;
+    p.split = 1; p.finish_rq = 4;
+    p.grp_seg = d.seg; p.grp_tiles = d.tiles; p.grp_ntiles = d.ntiles; p.grp_b = d.B;
+
+    // digits: what these operands needed last time, else the widest the 32-row kernels have (the launch is bound
+    // by the weight stream, not by the MFMA count)
+    const OperandKey key_a(d.A, (long)d.rows, d.K, 8), key_b(d.B, (long)d.groups * d.N, d.K, d.b32 ? 4 : 8);
+    int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
+    if (!na) {
+        auto it = g_cache.partner_a.find(key_b);
+        na = it != g_cache.partner_a.end() ? it->second : 5;
+    }
+    if (!nb) nb = 5;
+
+    for (int attempt = 0; attempt < 3; attempt++) {
+        const Instance *inst = pick_instance(na, nb, d.b32 != 0, true);
+        if (!inst) return 1;
+        MfmaKernel fn = inst->fn[d.b32 ? kB32Group : kB64Group];
+        if (!fn) return 1;
+        const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
+        const int ksteps = (d.K + 31) / 32;
+        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return 1;
+        p.tiles_n = (d.N + inst->bn - 1) / inst->bn;
+        const long max_mtiles = (long)d.rows / 32 + d.groups;
+        const long blocks = max_mtiles * p.tiles_n;
+        if (blocks > 0x7FFFFFFFL / 8) return 1;
+        p.main_tiles = (int)blocks;
+        if (!grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return zk_last_error() != kOk ? -1 : 1;
+        p.wg_range = g_cache.wg;
+        const size_t lds = 2 * (size_t)inst->kk * ((inst->bm / 32) * inst->na + (inst->bn / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
+        static std::set<const void *> lds_raised;
+        if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
+            if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+                set_error(kLaunchFailure, "grouped gemm: cannot raise the LDS limit to %zu bytes", lds);
+                return -1;
+            }
+            lds_raised.insert((const void *)fn);
+        }
+        fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
+        {
+            const hipError_t err = hipGetLastError();
+            if (err != hipSuccess) {
+                set_error(kLaunchFailure, "grouped gemm: launch failed (%s; digits %d,%d, %ld workgroups)", hipGetErrorString(err), inst->na, inst->nb, blocks);
+                return -1;
+            }
+        }
+        range_fold_kernel<<<1, 256, 0, 0>>>(nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr);
+        int64_t r[4];
+        if (!read_range(p.range, r)) { set_error(kLaunchFailure, "grouped gemm: range readback failed"); return -1; }
+        const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
+        g_cache.store_pair(key_a, need_a, key_b, need_b);
+        *limbs_a = inst->na;
+        *limbs_b = inst->nb;
+        if (need_a <= inst->na && need_b <= inst->nb) return 0;
+        na = need_a;
+        nb = need_b;
+    }
+    set_error(kLaunchFailure, "grouped gemm: digit count did not settle");
+    return -1;
 }
 
 }  // namespace zk

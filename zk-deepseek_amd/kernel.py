@@ -66,9 +66,14 @@ lib.zk_gemm_get_path.restype = _ci
 lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
 lib.zk_timer_stop_ms.restype = ctypes.c_float
 lib.zk_gemm_guard_hits.restype = ctypes.c_long
+lib.zk_gemm_grouped_mfma_calls.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
 lib.gate_route_q23.argtypes = [_vp] * 5 + [_ci] * 5
+lib.moe_dispatch.argtypes = [_vp, _ci, _ci, _ci] + [_vp] * 6
+lib.moe_gather_rows.argtypes = [_vp, _vp, _vp, _ci, _ci]
+lib.int64_grouped_bmm_launcher.argtypes = [_vp, _vp, _ci, _vp, _vp, ctypes.c_longlong, _vp, _vp, _vp, _ci, _ci, _ci, _ci]
+lib.moe_combine.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]
 lib.zk_dump_device.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
 lib.zk_dump_host.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
 lib.zk_dump_flush.restype = ctypes.c_long
@@ -361,6 +366,77 @@ def gate_route(scores, bias, n_groups, topk_groups, topk, raw_weights=None):
                        0 if raw_weights is None else raw_weights.data_ptr(), T, E, n_groups, topk_groups, topk)
     _check("gate_route_q23")
     return weights, indices
+
+
+# ---- MoE dispatch on the device (replaces the Python loop over the experts of MoE.forward, model.py:1325-1383)
+def pointer_table(tensors):
+    """device array with the addresses of the experts' weight matrices (keep the tensors alive while it is used)"""
+    return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device="cuda")
+
+
+def moe_dispatch(indices, n_experts):
+    """indices [T,K] int64 -> dict of int32 device tensors: seg [E+1], token [T*K], pos [T,K], tiles, ntiles"""
+    assert indices.is_cuda and indices.dtype == torch.int64 and indices.is_contiguous() and indices.dim() == 2
+    T, K = indices.shape
+    i32 = lambda n: torch.empty((n,), dtype=torch.int32, device=indices.device)
+    d = {"seg": i32(n_experts + 1), "token": i32(T * K), "pos": i32(T * K), "tiles": i32(2 * (T * K // 32 + n_experts)),
+         "ntiles": i32(1), "rows": T * K, "groups": n_experts}
+    counts = i32(n_experts)
+    lib.moe_dispatch(indices.data_ptr(), T, K, n_experts, counts.data_ptr(), d["seg"].data_ptr(), d["token"].data_ptr(),
+                     d["pos"].data_ptr(), d["tiles"].data_ptr(), d["ntiles"].data_ptr())
+    _check("moe_dispatch")
+    d["pos"] = d["pos"].view(T, K)
+    return d
+
+
+def moe_gather_rows(x, disp):
+    """x [T,N] int64 -> [T*K,N]: the rows of x in the sorted (by expert) order of `disp`"""
+    assert x.is_cuda and x.dtype == torch.int64 and x.is_contiguous() and x.dim() == 2
+    out = torch.empty((disp["rows"], x.shape[1]), dtype=torch.int64, device=x.device)
+    lib.moe_gather_rows(x.data_ptr(), disp["token"].data_ptr(), out.data_ptr(), disp["rows"], x.shape[1])
+    _check("moe_gather_rows")
+    return out
+
+
+def int64_grouped_bmm(A, b_table, b32, N, c_rescale, disp, want_remainder=False):
+    """A [rows,K] int64 sorted by expert, b_table = pointer_table(weights [N,K]) -> C [rows,N] (and R): every expert's
+    segment of rows times that expert's matrix, with the semantics of int64_bmm_broadcast per segment"""
+    assert A.is_cuda and A.dtype == torch.int64 and A.is_contiguous() and A.shape[0] == disp["rows"]
+    assert b_table.is_cuda and b_table.dtype == torch.int64 and b_table.numel() == disp["groups"]
+    rows, Kd = A.shape
+    C = torch.empty((rows, N), dtype=torch.int64, device=A.device)
+    R = torch.empty((rows, N), dtype=torch.int64, device=A.device) if want_remainder else None
+    lib.int64_grouped_bmm_launcher(A.data_ptr(), b_table.data_ptr(), 1 if b32 else 0, C.data_ptr(), 0 if R is None else R.data_ptr(),
+                                   c_rescale, disp["seg"].data_ptr(), disp["tiles"].data_ptr(), disp["ntiles"].data_ptr(),
+                                   disp["groups"], rows, Kd, N)
+    _check("int64_grouped_bmm")
+    return (C, R) if want_remainder else C
+
+
+def moe_combine(ye, weights, disp, T, shift=23):
+    """ye [T*K,N] expert outputs in sorted order, weights [T,K] -> y [T,N] = sum_k (ye[pos[t,k]] * weights[t,k]) >> shift"""
+    assert ye.is_cuda and weights.is_cuda and ye.is_contiguous() and weights.is_contiguous() and weights.dtype == torch.int64
+    K = weights.shape[1]
+    y = torch.empty((T, ye.shape[1]), dtype=torch.int64, device=ye.device)
+    lib.moe_combine(ye.data_ptr(), weights.data_ptr(), disp["pos"].data_ptr(), y.data_ptr(), T, K, ye.shape[1], shift)
+    _check("moe_combine")
+    return y
+
+
+def moe_experts(x, weights, indices, w1_table, w3_table, w2_table, b32, inter, c13, c2):
+    """The routed-expert part of MoE.forward (inference/model.py:1355-1381) without the Python loop: x [T,dim] Q23
+    activations, (weights, indices) from the gate, pointer tables of the experts' w1/w3 [inter,dim] and w2 [dim,inter]
+    -> y [T,dim] = sum over each token's experts of (w2 . ((silu(w1 . x) * (w3 . x)) >> 23) * weight) >> 23."""
+    T, dim = x.shape
+    E = w1_table.numel()
+    disp = moe_dispatch(indices.contiguous(), E)
+    xs = moe_gather_rows(x.contiguous(), disp)
+    g = int64_grouped_bmm(xs, w1_table, b32, inter, c13, disp)
+    u = int64_grouped_bmm(xs, w3_table, b32, inter, c13, disp)
+    h = torch.empty_like(g)
+    silu_mul_q23(g.unsqueeze(0), u.unsqueeze(0), h.unsqueeze(0))
+    ye = int64_grouped_bmm(h, w2_table, b32, dim, c2, disp)
+    return moe_combine(ye, weights.contiguous(), disp, T)
 
 
 def silu_mul_q23(R, U, C, S=None):
