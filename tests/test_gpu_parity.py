@@ -104,6 +104,24 @@ def test_gemm_operand_divisors(K, oracle, path):
         _gemm_case(K, oracle, path, A, W, a_rs, b_rs, 21)
 
 
+@pytest.mark.parametrize("w32", [False, True])
+@pytest.mark.parametrize("b_rs", [2, 256, 1 << 20, 1 << 40, 1 << 62])
+def test_gemm_head_projection_divisor_on_mfma(K, oracle, w32, b_rs):
+    """the head's shape in small: one to a few rows against many columns, weights divided by a power of two before the
+    product (inference/model.py:1519).  Truncation toward zero matters for the negative weights; the 32-row MFMA
+    kernels fold the division into their digit split, more rows go to the vector-ALU kernel's shift path."""
+    rng = np.random.default_rng(b_rs % 1000 + w32)
+    W = rand_i32(rng, (700, 320), 31) if w32 else rand_i64(rng, (700, 320), 45)
+    W[0, :6] = [-256, -255, -257, 255, 256, -1]
+    K.lib.zk_gemm_set_path(0)
+    for M in (1, 7, 32, 40):
+        A = rand_i64(rng, (1, M, 320), 36)
+        for _ in range(2):                                     # the second call runs on the remembered digit counts
+            _gemm_case(K, oracle, 0, A, W, 1, b_rs, 21)
+        mfma_expected = M <= 32 and (w32 or b_rs >= 256)        # 45-bit weights / 2 still need six digits
+        assert (K.gemm_last_plan()[0] == 2) == mfma_expected, (M, K.gemm_last_plan())
+
+
 def test_gemm_rejects_bad_arguments(K):
     A = torch.zeros((1, 2, 3), dtype=torch.int64, device="cuda")
     W = torch.zeros((4, 3), dtype=torch.int64, device="cuda")

@@ -71,6 +71,7 @@ struct MfmaParams {
     const int *grp_tiles;           // [2 * tiles] group and first row of every 32-row tile
     const int *grp_ntiles;          // how many of them exist (the grid is sized for the worst case)
     const void *const *grp_b;       // [groups] B of every group
+    int b_shift;                    // BRS kernels: every element of B is divided by 2^b_shift first, truncating toward zero
     int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
 };
 
@@ -140,6 +141,13 @@ __host__ __device__ static inline int limbs_needed(int64_t lo, int64_t hi)
     return 9;
 }
 
+// C++ division by 2^s (truncation toward zero) as shifts: the bias makes the arithmetic shift round negative values up
+__device__ __forceinline__ int64_t tdiv_pow2(int64_t x, int s)
+{
+    const uint64_t bias = (uint64_t)(x >> 63) & (((uint64_t)1 << s) - 1);
+    return (int64_t)((uint64_t)x + bias) >> s;
+}
+
 // ---- range tracking ------------------------------------------------------------------------------
 struct MinMax { int64_t lo, hi; };
 
@@ -201,6 +209,7 @@ __global__ __launch_bounds__(256) void range_sample_kernel(MfmaParams p, int b32
                     long off = (long)g * p.sB + row * p.ldbn + k * p.ldbk;
                     v = b32 ? (int64_t)reinterpret_cast<const int32_t *>(p.B)[off]
                             : reinterpret_cast<const int64_t *>(p.B)[off];
+                    v = tdiv_pow2(v, p.b_shift);
                 }
                 mm_update(r, v);
             }
@@ -372,7 +381,7 @@ __global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long lon
 // outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
 // own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
 // to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
-template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false>
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 {
     constexpr int T = 64 * WVM * WVN;
@@ -566,7 +575,14 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
         for (int it = 0; it < B_IT; it++) {
             uint2 dg[NB];
-            limb_split8<NB>(sb[it], dg);
+            if (BRS) {
+                int64_t y[8];
+#pragma unroll
+                for (int q = 0; q < 8; q++) y[q] = tdiv_pow2(sb[it][q], p.b_shift);
+                limb_split8<NB>(y, dg);
+            } else {
+                limb_split8<NB>(sb[it], dg);
+            }
 #pragma unroll
             for (int i = 0; i < NB; i++)
                 *reinterpret_cast<uint2 *>(smem + b_dst[it] + buf * b_stride[it] + i * 1024) = dg[i];
@@ -632,7 +648,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
             for (int it = 0; it < B_IT; it++)
 #pragma unroll
-                for (int q = 0; q < 8; q++) mm_update(rb, sb[it][q]);
+                for (int q = 0; q < 8; q++) mm_update(rb, BRS ? tdiv_pow2(sb[it][q], p.b_shift) : sb[it][q]);     // what the digits are taken from
         }
     };
 
@@ -805,7 +821,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
 typedef void (*MfmaKernel)(MfmaParams);
 typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
 
-enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kVariants };
+enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kB64FlyRs, kB32FlyRs, kVariants };
 
 struct Instance {
     int na, nb, bm, bn, threads, kk;
@@ -843,6 +859,9 @@ static Instance make_instance()
     if constexpr (SKINNY) {          // grouped launches (one B per segment of rows) run on the 32-row tiles only
         s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true>;
         if constexpr (NB <= 5) s.fn[kB32Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, true>;
+        // and so do products whose B is divided by a power of two first (the model's head projection)
+        s.fn[kB64FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, true>;
+        if constexpr (NB <= 5) s.fn[kB32FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, true>;
     }
     s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
     s.planes[0] = a_planes_kernel<NA, 2, KK>;
@@ -1003,7 +1022,14 @@ static bool init_cache()
 
 bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
 {
-    if (d.a_rs != 1 || d.b_rs != 1) return false;                    // operand divisors: VALU path
+    // Operand divisors: a power of two on B is folded into the digit split of the 32-row kernels (the head projection
+    // divides its weights by 256, inference/model.py:1519, and runs on the last token only); anything else: VALU path.
+    int b_shift = 0;
+    if (d.a_rs != 1) return false;
+    if (d.b_rs != 1) {
+        if (d.b_rs <= 0 || (d.b_rs & (d.b_rs - 1)) != 0 || d.M > 32) return false;
+        while (((int64_t)1 << b_shift) < d.b_rs) b_shift++;
+    }
     if (d.K <= 0 || d.M <= 0 || d.N <= 0 || d.G <= 0) return false;
     if (d.G > 65535) return false;
     const bool kmajor = d.ldbn == 1 && d.ldbk != 1;
@@ -1011,14 +1037,16 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     if (!init_cache()) return false;
     drain_pending();
 
-    MfmaParams p;
+    MfmaParams p = {};
     p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
     p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift; p.init = d.init;
     p.range = g_cache.dev;
     p.verify_b_all_batches = d.sB != 0;
+    p.b_shift = b_shift;
 
-    const OperandKey key_a(d.A, (long)d.G * d.M, d.K, 8), key_b(d.B, d.N, d.K, d.b32 ? 4 : 8);
+    // (a divided B has another range than the raw one: the shift is part of its key)
+    const OperandKey key_a(d.A, (long)d.G * d.M, d.K, 8), key_b(d.B, d.N, d.K, (d.b32 ? 4 : 8) | (b_shift << 8));
     int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
     // Activations gathered into a fresh buffer for a known weight matrix (the experts of a MoE layer): guess the
     // digits the last activations multiplied with that matrix needed.  A wrong guess costs one guarded recomputation.
@@ -1061,7 +1089,9 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass (never for the
         // 32-row tiles: splitting a handful of rows on the fly is cheaper than another kernel in front)
         const bool use_planes = !kmajor && p.tiles_n >= 4 && !inst->skinny;
-        const int variant = kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
+        if (b_shift && (kmajor || !inst->skinny)) return false;
+        const int variant = b_shift ? (d.b32 ? kB32FlyRs : kB64FlyRs)
+                          : kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
         if (!fn) return false;
@@ -1080,6 +1110,14 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             if (total < g_cache.cus) {
                 tail = (int)total;
                 split = g_cache.cus / tail;
+                if (split > 64) split = 64;
+                if (split > steps / 4) split = steps / 4;
+                p.finish_rq = 16;
+            } else if (inst->skinny && total < 8L * g_cache.cus) {
+                // a few rows against many columns is a weight stream: more, shorter workgroups keep more of it in
+                // flight and even out the last round (the partial sums of so few rows cost next to nothing)
+                tail = (int)total;
+                split = (int)((8L * g_cache.cus + total - 1) / total);
                 if (split > 64) split = 64;
                 if (split > steps / 4) split = steps / 4;
                 p.finish_rq = 16;

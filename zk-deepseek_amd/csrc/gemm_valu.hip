@@ -23,6 +23,7 @@ struct ValuParams {
     long lda, sA, ldbn, ldbk, sB, ldc, sC;
     int M, N, K, shift;
     int64_t init, a_rs, b_rs;
+    int a_shift, b_shift;                     // log2 of a divisor that is a positive power of two, else -1
     int tiles_m, tiles_n;
     long tiles;                               // tiles_m * tiles_n * G, walked by a 1-D grid
     const unsigned long long *guard;          // when set: do nothing unless *guard != 0
@@ -32,6 +33,16 @@ template <bool B32>
 __device__ __forceinline__ int64_t load_b(const void *B, long off)
 {
     return B32 ? (int64_t)reinterpret_cast<const int32_t *>(B)[off] : reinterpret_cast<const int64_t *>(B)[off];
+}
+
+// operand / divisor as C++ computes it; divisors that are powers of two (the model's only ones: 1 and 256) are shifts
+__device__ __forceinline__ int64_t rescale_operand(int64_t v, int64_t rs, int shift)
+{
+    if (shift >= 0) {
+        const uint64_t bias = (uint64_t)(v >> 63) & (((uint64_t)1 << shift) - 1);
+        return (int64_t)((uint64_t)v + bias) >> shift;
+    }
+    return tdiv64(v, rs);
 }
 
 template <bool B32, bool KMAJOR, bool RESCALE>
@@ -67,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(ValuParams p)
         for (int i = 0; i < 4; i++) {
             int m = m0 + lrow, k = k0 + lk + i;
             int64_t v = (m < p.M && k < p.K) ? Ag[(long)m * p.lda + k] : 0;
-            ra[i] = RESCALE ? tdiv64(v, p.a_rs) : v;
+            ra[i] = RESCALE ? rescale_operand(v, p.a_rs, p.a_shift) : v;
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -75,7 +86,7 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(ValuParams p)
             if (KMAJOR) { n = n0 + ln + i; k = k0 + kk_b; }
             else { n = n0 + lrow; k = k0 + lk + i; }
             int64_t v = (n < p.N && k < p.K) ? load_b<B32>(p.B, boff + (long)n * p.ldbn + (long)k * p.ldbk) : 0;
-            rb[i] = RESCALE ? tdiv64(v, p.b_rs) : v;
+            rb[i] = RESCALE ? rescale_operand(v, p.b_rs, p.b_shift) : v;
         }
     };
 
@@ -134,6 +145,14 @@ void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard)
     p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift;
     p.init = d.init; p.a_rs = d.a_rs; p.b_rs = d.b_rs;
+    auto log2_exact = [](int64_t v) {
+        if (v <= 0 || (v & (v - 1)) != 0) return -1;
+        int s = 0;
+        while (((int64_t)1 << s) < v) s++;
+        return s;
+    };
+    p.a_shift = log2_exact(d.a_rs);
+    p.b_shift = log2_exact(d.b_rs);
     p.tiles_m = (d.M + kVT - 1) / kVT;
     p.tiles_n = (d.N + kVT - 1) / kVT;
     p.tiles = (long)p.tiles_m * p.tiles_n * d.G;
