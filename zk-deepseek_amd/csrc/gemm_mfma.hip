@@ -319,23 +319,31 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
 
 // Folds the per-workgroup ranges of the plane pre-pass (`mm`, A only) and of the GEMM kernel (`wg`, A and B) into
 // range[0..3] and leaves the verdict in range[4]: 0 when `na` and `nb` digits covered them, 1 otherwise.
-// `host_copy`, when set, is pinned host memory that receives the same five words.
-__global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long long *mm, long mm_count,
-                                                         const unsigned long long *wg, long wg_count,
-                                                         unsigned long long *range, int na, int nb,
-                                                         unsigned long long *host_copy)
+// `host_copy`, when set, is pinned host memory that receives the same five words.  One workgroup of any size.
+struct FoldArgs {
+    const unsigned long long *mm;
+    long mm_count;
+    const unsigned long long *wg;
+    long wg_count;
+    unsigned long long *range;
+    int na, nb;
+    unsigned long long *host_copy;
+};
+
+__device__ __forceinline__ void range_fold_body(const FoldArgs &f)
 {
-    __shared__ unsigned long long red[4][4];
+    __shared__ unsigned long long red[16][4];
+    const int nthreads = blockDim.x;
     unsigned long long v[4] = { ~0ull, 0ull, ~0ull, 0ull };
-    for (long i = threadIdx.x; i < mm_count; i += 256) {
-        const unsigned long long a = mm[2 * i], b = mm[2 * i + 1];
+    for (long i = threadIdx.x; i < f.mm_count; i += nthreads) {
+        const unsigned long long a = f.mm[2 * i], b = f.mm[2 * i + 1];
         v[0] = a < v[0] ? a : v[0];
         v[1] = b > v[1] ? b : v[1];
     }
-    for (long i = threadIdx.x; i < wg_count; i += 256) {
+    for (long i = threadIdx.x; i < f.wg_count; i += nthreads) {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const unsigned long long a = wg[4 * i + q];
+            const unsigned long long a = f.wg[4 * i + q];
             v[q] = (q & 1) ? (a > v[q] ? a : v[q]) : (a < v[q] ? a : v[q]);
         }
     }
@@ -353,25 +361,27 @@ __global__ __launch_bounds__(256) void range_fold_kernel(const unsigned long lon
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; w++)
+        for (int w = 1; w < nthreads / 64; w++)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const unsigned long long o = red[w][q];
                 v[q] = (q & 1) ? (o > v[q] ? o : v[q]) : (o < v[q] ? o : v[q]);
             }
 #pragma unroll
-        for (int q = 0; q < 4; q++) range[q] = v[q];
+        for (int q = 0; q < 4; q++) f.range[q] = v[q];
         const int need_a = limbs_needed((int64_t)(v[0] ^ kSignFlip), (int64_t)(v[1] ^ kSignFlip));
         const int need_b = limbs_needed((int64_t)(v[2] ^ kSignFlip), (int64_t)(v[3] ^ kSignFlip));
-        const unsigned long long verdict = (need_a <= na && need_b <= nb) ? 0ull : 1ull;
-        range[4] = verdict;
-        if (host_copy) {
+        const unsigned long long verdict = (need_a <= f.na && need_b <= f.nb) ? 0ull : 1ull;
+        f.range[4] = verdict;
+        if (f.host_copy) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) host_copy[q] = v[q];
-            host_copy[4] = verdict;
+            for (int q = 0; q < 4; q++) f.host_copy[q] = v[q];
+            f.host_copy[4] = verdict;
         }
     }
 }
+
+__global__ __launch_bounds__(256) void range_fold_kernel(FoldArgs f) { range_fold_body(f); }
 
 // ---- the GEMM kernel -------------------------------------------------------------------------------
 // WVM x WVN waves per workgroup, WM x WN 32x32 MFMA tiles per wave, KK MFMA k-depths (32 k each) per pipeline
@@ -766,9 +776,14 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
 // Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
 // Thread layout and element order are those of the GEMM kernel's epilogue.
+// The workgroup behind the last one folds the ranges (the GEMM kernel has left them by then), which saves a launch.
 template <int WVM, int WVN, int WM, int WN>
-__global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaParams p)
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaParams p, FoldArgs fold)
 {
+    if (blockIdx.x == gridDim.x - 1) {
+        range_fold_body(fold);
+        return;
+    }
     constexpr int T = 64 * WVM * WVN, BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WVN, wn = wave % WVN;
@@ -793,7 +808,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
                 const long qs = (long)(T / 64) * (WM * WN * 16);          // from one slice to the next
                 if (p.part64) {
                     uint64_t s = 0;
-#pragma unroll 8
+#pragma unroll 16
                     for (int sidx = 0; sidx < p.split; sidx++) s += p.partials[(q0 + sidx * qs) * 64 + lane];
                     const uint64_t t = lo + s;
                     hi += (uint64_t)((int64_t)s >> 63) + (t < lo ? 1 : 0);
@@ -819,6 +834,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
 
 // ---- host side ---------------------------------------------------------------------------------------
 typedef void (*MfmaKernel)(MfmaParams);
+typedef void (*FinishKernel)(MfmaParams, FoldArgs);
 typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
 
 enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kB64FlyRs, kB32FlyRs, kVariants };
@@ -828,7 +844,7 @@ struct Instance {
     bool skinny;                 // 32-row tiles for M <= 32
     MfmaKernel fn[kVariants];
     PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
-    MfmaKernel finish;           // adds up the partial sums of split tail tiles
+    FinishKernel finish;         // adds up the partial sums of split tail tiles (and folds the ranges)
 };
 
 
@@ -1176,12 +1192,13 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                 return false;
             }
         }
+        const FoldArgs fold = { g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb, slot ? slot->host : nullptr };
         if (p.split > 1) {
-            inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq)), dim3((unsigned)inst->threads), 0, 0>>>(p);
+            inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq + 1)), dim3((unsigned)inst->threads), 0, 0>>>(p, fold);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
+        } else {
+            range_fold_kernel<<<1, 256, 0, 0>>>(fold);
         }
-        range_fold_kernel<<<1, 256, 0, 0>>>(g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb,
-                                            slot ? slot->host : nullptr);
         *limbs_a = inst->na;
         *limbs_b = inst->nb;
         if (slot) {
@@ -1267,7 +1284,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
                 return -1;
             }
         }
-        range_fold_kernel<<<1, 256, 0, 0>>>(nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr);
+        range_fold_kernel<<<1, 256, 0, 0>>>(FoldArgs{ nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr });
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "grouped gemm: range readback failed"); return -1; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
