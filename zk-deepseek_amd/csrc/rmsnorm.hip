@@ -26,12 +26,38 @@ __device__ __forceinline__ void u192_add(U192 &a, const U192 &b)
     a.w2 = a.w2 + b.w2 + c1;
 }
 
-__device__ __forceinline__ void u192_add_square(U192 &a, int64_t v)
-{
-    u128 sq = (u128)((i128)v * (i128)v);
-    U192 b = { (uint64_t)sq, (uint64_t)(sq >> 64), 0 };
-    u192_add(a, b);
-}
+// Per-thread sum of squares with three multiplies per element: for m = |v| = hi * 2^32 + lo,
+//   m^2 = lo*lo + 2^33 * lo*hi + 2^64 * hi*hi,
+// and each of the three products is summed in its own 64-bit column with a carry counter; the columns are merged
+// once per thread.  (The compiler's 128-bit square of a sign-extended value costs three times the multiplies.)
+struct SquareSum {
+    uint64_t ll = 0, lh = 0, hh = 0;
+    uint32_t cll = 0, clh = 0, chh = 0;
+    __device__ __forceinline__ void add(int64_t v)
+    {
+        const uint64_t m = v < 0 ? 0 - (uint64_t)v : (uint64_t)v;
+        const uint32_t lo = (uint32_t)m, hi = (uint32_t)(m >> 32);
+        uint64_t t = ll + (uint64_t)lo * lo;
+        cll += t < ll;
+        ll = t;
+        t = lh + (uint64_t)lo * hi;
+        clh += t < lh;
+        lh = t;
+        t = hh + (uint64_t)hi * hi;
+        chh += t < hh;
+        hh = t;
+    }
+    __device__ __forceinline__ U192 total() const
+    {
+        U192 r = { ll, cll, 0 };                                               // ll + 2^64 cll
+        // (lh + 2^64 clh) * 2^33
+        const U192 mid = { lh << 33, (lh >> 31) | ((uint64_t)clh << 33), (uint64_t)clh >> 31 };
+        u192_add(r, mid);
+        const U192 top = { 0, hh, chh };                                       // (hh + 2^64 chh) * 2^64
+        u192_add(r, top);
+        return r;
+    }
+};
 
 __device__ __forceinline__ U192 wave_sum_u192(U192 a)
 {
@@ -173,9 +199,9 @@ __global__ __launch_bounds__(kRmsThreads) void rms_stat_kernel(const int64_t *__
 {
     __shared__ U192 red[kRmsThreads / 64];
     const int64_t *a = A + (long)blockIdx.x * N;
-    U192 acc = { 0, 0, 0 };
-    for (int i = threadIdx.x; i < N; i += kRmsThreads) u192_add_square(acc, a[i]);
-    U192 tot = block_sum_u192<kRmsThreads>(acc, red);
+    SquareSum sq;
+    for (int i = threadIdx.x; i < N; i += kRmsThreads) sq.add(a[i]);
+    U192 tot = block_sum_u192<kRmsThreads>(sq.total(), red);
     if (threadIdx.x == 0) rms[blockIdx.x] = rms_finalize(tot, eps, dim);
 }
 
@@ -239,7 +265,7 @@ __global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__res
     const long row = blockIdx.x;
     const int64_t *a = A + row * N;
     int64_t v[EPT];
-    U192 acc = { 0, 0, 0 };
+    SquareSum sq;
     if (VEC) {
 #pragma unroll
         for (int j = 0; j < EPT / 2; j++) {
@@ -248,18 +274,18 @@ __global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__res
                 const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
                 v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
                 v[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
-                u192_add_square(acc, v[2 * j]);
-                u192_add_square(acc, v[2 * j + 1]);
+                sq.add(v[2 * j]);
+                sq.add(v[2 * j + 1]);
             }
         }
     } else {
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
             const int i = j * THREADS + threadIdx.x;
-            if (i < N) { v[j] = a[i]; u192_add_square(acc, v[j]); }
+            if (i < N) { v[j] = a[i]; sq.add(v[j]); }
         }
     }
-    U192 tot = block_sum_u192<THREADS>(acc, red);
+    U192 tot = block_sum_u192<THREADS>(sq.total(), red);
     if (threadIdx.x == 0) {
         int64_t r = rms_finalize(tot, eps, dim);
         rms_s = r;
