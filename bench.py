@@ -76,7 +76,7 @@ def gemm_leg(K, A, W, c, steps, warmup):
     path, la, lb = K.gemm_last_plan()
     macs = Bd * M * N * Kd
     return {"ms": ms, "gmacs": macs / ms / 1e6, "macs": macs, "path": {1: "valu", 2: "mfma_i8"}.get(path, "?"),
-            "limbs_a": la, "limbs_b": lb}
+            "limbs_a": la, "limbs_b": lb, "digit_pairs": K.gemm_last_pairs()}
 
 
 def main():
@@ -158,6 +158,8 @@ def main():
         Af = full_range(g4, (1, M, Kd)).cuda()
         Wf = full_range(g4, (N, Kd)).cuda()
         extra["gemm_config4_full_range"] = gemm_leg(K, Af, Wf, 29, max(3, args.steps // 4), 1)
+        # the same product modulo 2^64 (shift 0): only the digit pairs below 2^64 are multiplied
+        extra["gemm_config4_full_range_shift0"] = gemm_leg(K, Af, Wf, 0, max(3, args.steps // 4), 1)
         del Af, Wf
         # real-model operand widths: Q31 activations (|x| < 2^37), int32 weights
         Am = randint(g4, -(1 << 37), 1 << 37, (1, M, Kd)).cuda()

@@ -180,6 +180,10 @@ void zk_gemm_set_path(int path);
 int zk_gemm_get_path(void);
 /* What the last GEMM-like call used: path (1/2) and the limb counts of A and B (0 for the VALU path). */
 void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
+/* i8 digit products per int64 multiply-add in the last GEMM-like call (0 for the VALU path).  At most
+ * limbs_a * limbs_b; fewer when the stored bits [shift, shift + 64) of the sum lie below the weight of the top
+ * digit pairs, which are then not multiplied at all. */
+int zk_gemm_last_pairs(void);
 /* The MFMA path guesses how many base-256 digits the operands need and checks the guess on the device.  A call
  * whose operands (pointer, shape) were seen before does not wait for that check: a guarded vector-ALU launch
  * behind it recomputes the outputs if the guess was too small.  This returns how many calls so far needed that

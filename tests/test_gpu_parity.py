@@ -68,6 +68,28 @@ def test_gemm_ranges_and_shifts(K, oracle, path, bits_a, bits_w, w32, c):
     _gemm_case(K, oracle, path, A, W, 1, 1, c)
 
 
+@pytest.mark.parametrize("c", [0, 1, 8, 31, 32, 33, 40, 63])
+@pytest.mark.parametrize("bits_a,bits_w,w32", [(63, 63, False), (63, 31, True), (36, 63, False)])
+def test_gemm_many_digit_operands_at_every_shift(K, oracle, bits_a, bits_w, w32, c):
+    """Operands of up to nine digits: the MFMA path leaves out the digit pairs whose weight lies above the stored bits
+    [c, c + 64) of the sum (8, 12 or all diagonals), so shifts on both sides of each boundary are checked, with
+    values whose top digits are as large as they get."""
+    rng = np.random.default_rng(bits_a + bits_w + c)
+    A = rand_i64(rng, (1, 130, 520), bits_a)
+    W = rand_i32(rng, (200, 520), bits_w) if w32 else rand_i64(rng, (200, 520), bits_w)
+    lim_a, lim_w = (1 << bits_a) - 1, (1 << bits_w) - 1
+    A[0, 1, :] = np.where(np.arange(520) % 2 == 0, lim_a, -lim_a - 1)
+    W[3, :] = np.where(np.arange(520) % 3 == 0, -lim_w - 1, lim_w)
+    _gemm_case(K, oracle, 2, A, W, 1, 1, c)
+    _, la, lb = K.gemm_last_plan()
+    kept = 8 if c == 0 else (12 if c <= 32 else 16)
+    if (la, lb) == (9, 9):      # the other digit counts have no 12-diagonal instance
+        assert K.gemm_last_pairs() == sum(1 for i in range(9) for j in range(9) if i + j < kept)
+    elif c == 0:
+        assert K.gemm_last_pairs() == sum(1 for i in range(la) for j in range(lb) if i + j < 8)
+    K.lib.zk_gemm_set_path(0)
+
+
 @pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 1, 7, 1), (3, 5, 17, 9), (1, 64, 64, 64), (1, 65, 129, 63),
                                    (1, 128, 32, 256), (2, 33, 1000, 31), (1, 257, 96, 130)])

@@ -191,6 +191,7 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b)
 }
 
 long zk_gemm_guard_hits(void) { return zk::gemm_mfma_guard_hits(); }
+int zk_gemm_last_pairs(void) { return zk::g_last_path == zk::kPathMfma ? zk::gemm_mfma_last_pairs() : 0; }
 
 long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
 

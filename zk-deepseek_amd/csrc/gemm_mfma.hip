@@ -383,6 +383,21 @@ __device__ __forceinline__ void range_fold_body(const FoldArgs &f)
 
 __global__ __launch_bounds__(256) void range_fold_kernel(FoldArgs f) { range_fold_body(f); }
 
+// Number of digit pairs (i', j') with i' + j' < d that come before (i, j) in row order (i' < i, or i' == i and j' < j).
+__host__ __device__ constexpr int kept_pairs_before(int na, int nb, int d, int i, int j)
+{
+    int n = 0;
+    for (int r = 0; r < i && r < na; r++) {
+        const int row = d - r < 0 ? 0 : (d - r > nb ? nb : d - r);
+        n += row;
+    }
+    if (i < na) {
+        const int row = d - i < 0 ? 0 : (d - i > nb ? nb : d - i);
+        n += j < row ? j : row;
+    }
+    return n;
+}
+
 // ---- the GEMM kernel -------------------------------------------------------------------------------
 // WVM x WVN waves per workgroup, WM x WN 32x32 MFMA tiles per wave, KK MFMA k-depths (32 k each) per pipeline
 // step.  APL: A comes from pre-split digit planes (plain copy into LDS); otherwise it is split on the fly like B.
@@ -391,13 +406,16 @@ __global__ __launch_bounds__(256) void range_fold_kernel(FoldArgs f) { range_fol
 // outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
 // own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
 // to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
-template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false>
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false, int DMAX = 16>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 {
     constexpr int T = 64 * WVM * WVN;
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 32 * KK, OCTS = BK / 8;
     constexpr int RUN = B32 ? 4 : 2;
-    constexpr int D = (NA + NB - 1) > 16 ? 16 : (NA + NB - 1);     // diagonal 16 has weight 2^128: dropped
+    // Diagonal d carries weight 2^(8d).  Diagonal 16 (2^128) never matters; a launch whose shift + 64 result bits
+    // end below 2^(8 DMAX) leaves out the digit pairs of the diagonals from DMAX up as well.
+    constexpr int D = (NA + NB - 1) > DMAX ? DMAX : (NA + NB - 1);
+    static_assert(DMAX >= 8 && DMAX <= 16, "the low 64 bits of the sum need diagonals 0..7");
     constexpr int A_BLOCKS = (BM / 32) * NA, B_BLOCKS = (BN / 32) * NB;
     constexpr int SUBSTAGE = (A_BLOCKS + B_BLOCKS) * 1024;
     constexpr int STAGE = KK * SUBSTAGE;
@@ -613,7 +631,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             for (int j = 0; j < NB; j++)
                 fb[b][j] = *reinterpret_cast<const v4i *>(base + ((A_BLOCKS + (wn * WN + b) * NB + j) * 1024) + lane * 16);
     };
-    constexpr int MFMAS = WM * WN * NA * NB;
+    // the digit pairs (i, j) with i + j < D are numbered in row order; a slice issues those numbered LO..HI-1
+    constexpr int MFMAS = WM * WN * kept_pairs_before(NA, NB, D, NA, 0);
     auto mfma_slice = [&](auto lo_tag, auto hi_tag, const v4i (&fa)[WM][NA], const v4i (&fb)[WN][NB]) {
         constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
 #pragma unroll
@@ -624,7 +643,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                 for (int a = 0; a < WM; a++)
 #pragma unroll
                     for (int b = 0; b < WN; b++) {
-                        const int idx = ((i * NB + j) * WM + a) * WN + b;
+                        const int idx = (kept_pairs_before(NA, NB, D, i, j) * WM + a) * WN + b;
                         if (idx >= LO && idx < HI && i + j < D)
                             acc[a][b][i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a][i], fb[b][j], acc[a][b][i + j], 0, 0, 0);
                     }
@@ -842,16 +861,17 @@ enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32
 struct Instance {
     int na, nb, bm, bn, threads, kk;
     bool skinny;                 // 32-row tiles for M <= 32
+    int dmax;                    // diagonals from this one up are left out (16: none but the 2^128 one)
     MfmaKernel fn[kVariants];
     PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
     FinishKernel finish;         // adds up the partial sums of split tail tiles (and folds the ranges)
 };
 
 
-template <int NA, int NB, bool SKINNY = false>
+template <int NA, int NB, bool SKINNY = false, int DMAX = 16>
 static Instance make_instance()
 {
-    constexpr int DD = NA + NB - 1;
+    constexpr int DD = (NA + NB - 1) > DMAX ? DMAX : (NA + NB - 1);      // diagonals kept = accumulator sets
     static_assert(!SKINNY || DD <= 10, "skinny tiles keep two waves per SIMD");
     // narrow: 8 waves as 2x4, 64x32 per wave (128x128); mid: 8 waves as 4x2, 32x32 per wave (128x64);
     // wide: 4 waves as 2x2, 32x32 per wave (64x64, one wave per SIMD because of the accumulator count)
@@ -863,21 +883,22 @@ static Instance make_instance()
     Instance s;
     s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
     s.skinny = SKINNY;
+    s.dmax = DMAX;
     for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
-    s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false>;
-    s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true>;
-    s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false>;
+    s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, false, DMAX>;
+    s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX>;
+    s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false, false, false, DMAX>;
     if constexpr (NB <= 5) {          // int32 values never need more than five digits
-        s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false>;
-        s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true>;
-        s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false>;
+        s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, false, DMAX>;
+        s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true, false, false, DMAX>;
+        s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false, false, false, DMAX>;
     }
     if constexpr (SKINNY) {          // grouped launches (one B per segment of rows) run on the 32-row tiles only
-        s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true>;
-        if constexpr (NB <= 5) s.fn[kB32Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, true>;
+        s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX>;
+        if constexpr (NB <= 5) s.fn[kB32Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, true, false, DMAX>;
         // and so do products whose B is divided by a power of two first (the model's head projection)
-        s.fn[kB64FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, true>;
-        if constexpr (NB <= 5) s.fn[kB32FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, true>;
+        s.fn[kB64FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, true, DMAX>;
+        if constexpr (NB <= 5) s.fn[kB32FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, true, DMAX>;
     }
     s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
     s.planes[0] = a_planes_kernel<NA, 2, KK>;
@@ -896,13 +917,17 @@ static const Instance *instances(int *count)
         make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(),
         make_instance<9, 5>(), make_instance<5, 9>(), make_instance<9, 9>(),
         make_instance<3, 3, true>(), make_instance<5, 5, true>(),
+        // many-digit operands whose shift + 64 result bits end below 2^96 or 2^64: fewer digit pairs
+        make_instance<9, 9, false, 12>(), make_instance<9, 9, false, 8>(),
+        make_instance<9, 5, false, 8>(), make_instance<5, 9, false, 8>(),
 #endif
     };
     *count = (int)(sizeof(table) / sizeof(table[0]));
     return table;
 }
 
-static const Instance *pick_instance(int na, int nb, bool b32, bool skinny)
+// need_diag: the result's top bit is below 2^(8 need_diag), so diagonals from need_diag up cannot reach it
+static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int need_diag = 16)
 {
     int count;
     const Instance *t = instances(&count);
@@ -910,8 +935,9 @@ static const Instance *pick_instance(int na, int nb, bool b32, bool skinny)
     long best_cost = 0;
     for (int i = 0; i < count; i++) {
         if (t[i].na < na || t[i].nb < nb || t[i].skinny != skinny) continue;
+        if (t[i].dmax < 16 && t[i].dmax < need_diag) continue;
         if (b32 && !t[i].fn[kB32Fly]) continue;
-        long cost = (long)t[i].na * t[i].nb;
+        long cost = kept_pairs_before(t[i].na, t[i].nb, t[i].dmax, t[i].na, 0);     // MFMAs per 32x32x32 block
         if (!best || cost < best_cost) { best = &t[i]; best_cost = cost; }
     }
     return best;
@@ -1006,6 +1032,9 @@ static void drain_pending()
     }
 }
 
+static int g_last_pairs = 0;
+int gemm_mfma_last_pairs() { return g_last_pairs; }
+
 long gemm_mfma_guard_hits()
 {
     std::lock_guard<std::mutex> lock(g_cache.mu);
@@ -1088,8 +1117,10 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     }
 
     for (int attempt = 0; attempt < 3; attempt++) {
-        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true) : nullptr;
-        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false);
+        // the stored bits are [shift, shift + 64) of the sum (the remainder lies below them)
+        const int need_diag = (d.shift + 64 + 7) / 8;
+        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
+        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag);
         if (!inst) return false;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
@@ -1184,6 +1215,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             lds_raised.insert((const void *)fn);
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
+        g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
         {
             const hipError_t err = hipGetLastError();
             if (err != hipSuccess) {
@@ -1277,6 +1309,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
             lds_raised.insert((const void *)fn);
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
+        g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
         {
             const hipError_t err = hipGetLastError();
             if (err != hipSuccess) {

@@ -66,6 +66,7 @@ lib.zk_gemm_get_path.restype = _ci
 lib.zk_gemm_last_plan.argtypes = [ctypes.POINTER(_ci), ctypes.POINTER(_ci), ctypes.POINTER(_ci)]
 lib.zk_timer_stop_ms.restype = ctypes.c_float
 lib.zk_gemm_guard_hits.restype = ctypes.c_long
+lib.zk_gemm_last_pairs.restype = ctypes.c_int
 lib.zk_gemm_grouped_mfma_calls.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
@@ -87,6 +88,11 @@ def _check(what):
         msg = lib.zk_last_error_string().decode()
         lib.zk_clear_error()
         raise RuntimeError("%s failed (code %d): %s" % (what, code, msg))
+
+
+def gemm_last_pairs():
+    """i8 digit products per int64 multiply-add in the last GEMM-like call (0 on the VALU path)"""
+    return int(lib.zk_gemm_last_pairs())
 
 
 def gemm_last_plan():
