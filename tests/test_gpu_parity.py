@@ -426,6 +426,36 @@ def test_rmsnorm_reference_entry_points(K, oracle):
     assert K.int64_RMS0(dev(A[0]), 1, 300) == int(oracle.rms_stat(A[:1], 1, 300)[0])
 
 
+@pytest.mark.parametrize("w32", [True, False])
+@pytest.mark.parametrize("r", [3, 977, (1 << 31) - 1, (1 << 36) + 12345, (1 << 52) + 3, (1 << 61) + 5])
+def test_rmsnorm_quotients_next_to_integers(K, oracle, r, w32):
+    """a * w / r exactly on, one below and one above multiples of r, at quotients from 0 to beyond 2^49, both signs:
+    the cases a floating-point estimate of the quotient cannot settle and the exact tiers behind it must"""
+    rng = np.random.default_rng(r % 1000)
+    N = 1024
+    n = np.concatenate([np.arange(-8, 8), rng.integers(-(1 << 20), 1 << 20, 200), rng.integers(-(1 << 40), 1 << 40, 200),
+                        rng.integers(-(1 << 51), 1 << 51, 100), [(1 << 49) - 1, 1 << 49, -(1 << 49), (1 << 50) + 1]])
+    prods = []
+    for q in n.tolist():
+        for delta in (-1, 0, 1, r - 1, -(r - 1), r // 2):
+            p = q * r + delta
+            if -(1 << 63) <= p < (1 << 63):
+                prods.append(p)
+    prods = np.array(prods[: (len(prods) // N) * N], dtype=np.int64).reshape(-1, N)
+    M = prods.shape[0]
+    # w = 1: the product is a itself; w = -1 and a small factor exercise the sign and a genuine multiplication
+    for wv, A in ((1, prods), (-1, -np.maximum(prods, -(1 << 63) + 1)), (3, prods // 3)):
+        W = np.full((N,), wv, dtype=np.int32 if w32 else np.int64)
+        rms = np.full((M,), r, dtype=np.int64)
+        C = torch.empty((M, N), dtype=torch.int64, device="cuda")
+        fn = K.lib.rms_norm_32 if w32 else K.lib.rms_norm_64
+        Ad, Wd, rd = dev(A), dev(W), dev(rms)
+        fn(Ad.data_ptr(), Wd.data_ptr(), rd.data_ptr(), C.data_ptr(), M, N)
+        torch.cuda.synchronize()
+        K._check("rms_norm")
+        assert np.array_equal(host(C), oracle.rms_norm_apply(np.ascontiguousarray(A), W, rms))
+
+
 def test_rmsnorm_model_shape(K, oracle):
     """[256,7168] at residual-stream magnitudes (|x| up to ~2^37, Q31) with int32 Q21 weights"""
     g = torch.Generator(device="cpu").manual_seed(600)

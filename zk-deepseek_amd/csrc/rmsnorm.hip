@@ -140,45 +140,99 @@ __device__ int64_t rms_finalize(U192 acc, int64_t eps, int64_t dim)
 
 // floor(a * w / r) as the reference computes it: C++ division of the 128-bit product, minus one when the
 // remainder is negative (inference/int64_gemm.cu:314-322).  r == 0 gives 0.
-__device__ __noinline__ int64_t rms_apply_slow(int64_t a, int64_t w, int64_t r)
+// Written as a shift-and-subtract loop on the magnitudes: this is the rare last resort, and a compact loop keeps
+// its register needs (which every kernel that contains it would inherit) next to nothing.
+__device__ __forceinline__ int64_t rms_apply_slow(int64_t a, int64_t w, int64_t r)
 {
     if (r == 0) return 0;
-    i128 prod = (i128)a * (i128)w;
-    i128 qq = prod / (i128)r;
-    i128 rr = prod % (i128)r;
-    if (rr < 0) qq -= 1;
-    return (int64_t)(uint64_t)(u128)qq;
+    const i128 prod = (i128)a * (i128)w;
+    const bool pneg = prod < 0;
+    const u128 up = pneg ? (u128)0 - (u128)prod : (u128)prod;
+    const uint64_t ur = r < 0 ? 0 - (uint64_t)r : (uint64_t)r;
+    uint64_t qh = 0, ql = 0, plo = (uint64_t)up, phi = (uint64_t)(up >> 64);
+    uint64_t rem = 0;                 // stays below ur <= 2^63, so doubling it cannot overflow 64 bits
+#pragma unroll 1
+    for (int bit = 0; bit < 128; bit++) {
+        rem = (rem << 1) | (phi >> 63);
+        phi = (phi << 1) | (plo >> 63);
+        plo <<= 1;
+        qh = (qh << 1) | (ql >> 63);
+        ql <<= 1;
+        if (rem >= ur) { rem -= ur; ql |= 1; }
+    }
+    u128 uq = ((u128)qh << 64) | ql;
+    // C++ semantics: the quotient truncates toward zero and the remainder takes the sign of the product
+    u128 qq = (pneg != (r < 0)) ? (u128)0 - uq : uq;
+    if (pneg && rem != 0) qq -= 1;
+    return (int64_t)(uint64_t)qq;
 }
 
-// Fast exact path for 0 < r < 2^62 and |quotient| < 2^49.  The quotient is estimated in double precision from
-// the operands themselves: a, w and 1/r each carry a relative error of at most 2^-53 and so does each of the two
-// products, so the estimate is off by less than 2^49 * 5 * 2^-53 < 0.32 and, rounded to nearest, lands within
-// one of the floor.  The remainder, exact modulo 2^64, settles which; anything else takes the slow path.
-// The rounding and the conversion to an integer are one addition: for |x| < 2^51 the low bits of
-// x + 1.5 * 2^52 hold round(x) as a fixed-point number.
+// Three tiers, each exact where it answers.
+//
+// The quotient x = a*w/r is estimated in double precision from the operands themselves,
+// xd = fl(fl(fl(a) * fl(w)) * fl(1 / fl(r))): six roundings of relative size 2^-53 at most, so |xd - x| <= |x| * 2^-50.
+//
+// Quick tier: n = floor(xd) is floor(x) whenever xd lies further than m = |xd| * 2^-49 (twice the bound and more)
+// from both n and n + 1; a zero product is exact as it is.  This is all most elements ever run.
+//
+// Remainder tier, 0 < r < 2^62 and |x| < 2^49: the estimate is off by less than 2^49 * 2^-50 = 0.5, so rounded to
+// nearest it lands within one of the floor; the remainder a*w - q*r, exact modulo 2^64, settles which.  The rounding
+// and the conversion to an integer are one addition: for |x| < 2^51 the low bits of x + 1.5 * 2^52 hold round(x) as
+// a fixed-point number.
+//
+// Anything else is divided the long way (rms_apply_slow).
+template <typename WT>
+__device__ __forceinline__ int64_t rms_apply_quick(int64_t a, WT w, double inv_r, bool fast_r, bool &certain)
+{
+    const double xd = (double)a * (double)w * inv_r;
+    const double fl = floor(xd);
+    const double frac = xd - fl;                     // exact
+    const double m = fabs(xd) * 0x1p-49;             // >= 1 once |xd| >= 2^49: such elements are never certain
+    certain = fast_r && ((frac > m && 1.0 - frac > m) || xd == 0.0);
+    const double magic = 6755399441055744.0;
+    return (int64_t)((uint64_t)__double_as_longlong(fl + magic) - (uint64_t)__double_as_longlong(magic));
+}
+
+template <typename WT>
+__device__ __forceinline__ int64_t rms_apply_fast(int64_t a, WT w, int64_t r, double inv_r, bool fast_r, bool &ok)
+{
+    // straight-line code: estimate, remainder, one-step correction by selects; `ok` says whether the result stands
+    const double xd = (double)a * (double)w * inv_r;
+    const double magic = 6755399441055744.0;
+    // (unsigned arithmetic throughout: a wild estimate must wrap, not overflow, on its way to being rejected)
+    uint64_t q = (uint64_t)__double_as_longlong(xd + magic) - (uint64_t)__double_as_longlong(magic);
+    const uint64_t plo = (uint64_t)a * (uint64_t)(int64_t)w;
+    uint64_t rem = plo - q * (uint64_t)r;
+    const bool neg = (int64_t)rem < 0, big = !neg && (int64_t)rem >= r;
+    q += big ? 1ull : (neg ? ~0ull : 0ull);
+    rem += neg ? (uint64_t)r : (big ? 0 - (uint64_t)r : 0ull);
+    ok = fast_r && fabs(xd) < 562949953421312.0 && (int64_t)rem >= 0 && (int64_t)rem < r;
+    return (int64_t)q;
+}
+
 template <typename WT>
 __device__ __forceinline__ int64_t rms_apply_one(int64_t a, WT w, int64_t r, double inv_r, bool fast_r)
 {
-    if (fast_r) {
-        const double xd = (double)a * (double)w * inv_r;
-        if (fabs(xd) < 562949953421312.0) {
-            const double magic = 6755399441055744.0;
-            int64_t q = __double_as_longlong(xd + magic) - __double_as_longlong(magic);
-            const uint64_t plo = (uint64_t)a * (uint64_t)(int64_t)w;
-            int64_t rem = (int64_t)(plo - (uint64_t)q * (uint64_t)r);
-            if (rem < 0) { q--; rem += r; }
-            else if (rem >= r) { q++; rem -= r; }
-            if (rem >= 0 && rem < r) return q;
-        }
+    bool ok;
+    const int64_t q = rms_apply_fast(a, w, r, inv_r, fast_r, ok);
+    if (__builtin_expect(!ok, 0)) return rms_apply_slow(a, (int64_t)w, r);
+    return q;
+}
+
+// two consecutive weights in one load (the callers guarantee an even index and 16-byte aligned rows; the weight
+// vector itself is only assumed to be aligned to its element size, so int64 weights stay two loads)
+template <typename WT> struct WPair { WT x, y; };
+template <typename WT>
+__device__ __forceinline__ WPair<WT> load_w_pair(const WT *W, int i, bool w_vec)
+{
+    if (sizeof(WT) == 4 && w_vec) {
+        const uint2 t = *reinterpret_cast<const uint2 *>(W + i);
+        return { (WT)(int32_t)t.x, (WT)(int32_t)t.y };
     }
-    return rms_apply_slow(a, (int64_t)w, r);
+    return { W[i], W[i + 1] };
 }
 
 constexpr int kRmsThreads = 256;
-#ifndef ZK_RMS_T8K
-#define ZK_RMS_T8K 512
-#define ZK_RMS_E8K 16
-#endif
 
 template <int THREADS>
 __device__ __forceinline__ U192 block_sum_u192(U192 acc, U192 *red)
@@ -224,10 +278,16 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
     int64_t *c = C + row * N;
     if (VEC) {
         v4i_r t[kApplyEpt / 2];
+        WPair<WT> wp[kApplyEpt / 2];
+        const bool w_vec = ((uintptr_t)W & 7) == 0;
+        unsigned redo = 0;
 #pragma unroll
         for (int j = 0; j < kApplyEpt / 2; j++) {
             const int i = base + (j * kRmsThreads + threadIdx.x) * 2;
-            if (i < N) t[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
+            if (i < N) {
+                t[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
+                wp[j] = load_w_pair(W, i, w_vec);
+            }
         }
 #pragma unroll
         for (int j = 0; j < kApplyEpt / 2; j++) {
@@ -235,11 +295,24 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
             if (i < N) {
                 const int64_t v0 = (int64_t)(((uint64_t)(uint32_t)t[j][1] << 32) | (uint32_t)t[j][0]);
                 const int64_t v1 = (int64_t)(((uint64_t)(uint32_t)t[j][3] << 32) | (uint32_t)t[j][2]);
-                const int64_t c0 = rms_apply_one(v0, W[i], r, inv_r, fast_r);
-                const int64_t c1 = rms_apply_one(v1, W[i + 1], r, inv_r, fast_r);
+                bool ok0, ok1;
+                const int64_t c0 = rms_apply_quick(v0, wp[j].x, inv_r, fast_r, ok0);
+                const int64_t c1 = rms_apply_quick(v1, wp[j].y, inv_r, fast_r, ok1);
+                redo |= (ok0 ? 0u : 1u << (2 * j)) | (ok1 ? 0u : 2u << (2 * j));
                 const v4i_r o = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
                                   (int)(uint32_t)((uint64_t)c1 >> 32) };
                 __builtin_nontemporal_store(o, reinterpret_cast<v4i_r *>(c + i));
+            }
+        }
+        // rare: elements the quick tier could not settle go through the other two and are stored again
+        if (__builtin_expect(redo != 0, 0)) {
+#pragma unroll
+            for (int j = 0; j < kApplyEpt / 2; j++) {
+                const int i = base + (j * kRmsThreads + threadIdx.x) * 2;
+                const int64_t v0 = (int64_t)(((uint64_t)(uint32_t)t[j][1] << 32) | (uint32_t)t[j][0]);
+                const int64_t v1 = (int64_t)(((uint64_t)(uint32_t)t[j][3] << 32) | (uint32_t)t[j][2]);
+                if (redo & (1u << (2 * j))) c[i] = rms_apply_one(v0, wp[j].x, r, inv_r, fast_r);
+                if (redo & (2u << (2 * j))) c[i + 1] = rms_apply_one(v1, wp[j].y, r, inv_r, fast_r);
             }
         }
     } else {
@@ -255,8 +328,11 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
 // Long rows get more threads rather than more elements per thread: fewer registers mean more rows in flight per
 // compute unit, which is what hides the serial stretch (reduction, division, square root) in the middle.
 // VEC: N is even and the rows are 16-byte aligned: elements are moved two at a time with streaming accesses.
-template <typename WT, int THREADS, int EPT, bool VEC>
-__global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
+// WPE: waves per SIMD the register allocation must leave room for.  Rows of 4K-8K elements run three workgroups of
+// eight waves per compute unit (WPE 6, 80 registers): measured, a third row in flight is worth more than the few
+// registers spilled for it, a fourth is not.
+template <typename WT, int THREADS, int EPT, bool VEC, int WPE>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
                                                                 int64_t *__restrict__ rms, int64_t *__restrict__ C,
                                                                 int N, int64_t eps, int64_t dim)
 {
@@ -265,6 +341,8 @@ __global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__res
     const long row = blockIdx.x;
     const int64_t *a = A + row * N;
     int64_t v[EPT];
+    WPair<WT> wp[EPT / 2];          // the weights travel with the row: no load is left for after the barrier
+    const bool w_vec = ((uintptr_t)W & 7) == 0;
     SquareSum sq;
     if (VEC) {
 #pragma unroll
@@ -272,6 +350,7 @@ __global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__res
             const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
                 const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
+                wp[j] = load_w_pair(W, i, w_vec);
                 v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
                 v[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
                 sq.add(v[2 * j]);
@@ -296,15 +375,27 @@ __global__ __launch_bounds__(THREADS) void rms_fused_kernel(const int64_t *__res
     const bool fast_r = r > 0 && r < ((int64_t)1 << 62);
     const double inv_r = fast_r ? 1.0 / (double)r : 0.0;
     if (VEC) {
+        unsigned redo = 0;
 #pragma unroll
         for (int j = 0; j < EPT / 2; j++) {
             const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
-                const int64_t c0 = rms_apply_one(v[2 * j], W[i], r, inv_r, fast_r);
-                const int64_t c1 = rms_apply_one(v[2 * j + 1], W[i + 1], r, inv_r, fast_r);
+                bool ok0, ok1;
+                const int64_t c0 = rms_apply_quick(v[2 * j], wp[j].x, inv_r, fast_r, ok0);
+                const int64_t c1 = rms_apply_quick(v[2 * j + 1], wp[j].y, inv_r, fast_r, ok1);
+                redo |= (ok0 ? 0u : 1u << (2 * j)) | (ok1 ? 0u : 2u << (2 * j));
                 const v4i_r t = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
                                   (int)(uint32_t)((uint64_t)c1 >> 32) };
                 __builtin_nontemporal_store(t, reinterpret_cast<v4i_r *>(C + row * N + i));
+            }
+        }
+        // rare: elements the quick tier could not settle go through the other two and are stored again
+        if (__builtin_expect(redo != 0, 0)) {
+#pragma unroll
+            for (int j = 0; j < EPT / 2; j++) {
+                const int i = (j * THREADS + threadIdx.x) * 2;
+                if (redo & (1u << (2 * j))) C[row * N + i] = rms_apply_one(v[2 * j], wp[j].x, r, inv_r, fast_r);
+                if (redo & (2u << (2 * j))) C[row * N + i + 1] = rms_apply_one(v[2 * j + 1], wp[j].y, r, inv_r, fast_r);
             }
         }
     } else {
@@ -351,16 +442,16 @@ static void launch_fused(const char *name, const int64_t *A, const WT *W, int64_
     if (!rms_args_ok(name, A, W, rms, C, M, N) || !stat_args_ok(name, eps, dim)) return;
     const bool vec = N % 2 == 0 && (((uintptr_t)A | (uintptr_t)C) & 15) == 0;
     const dim3 grid((unsigned)M);
-#define ZK_RMS_LAUNCH(THREADS, EPT)                                                                                   \
-    do {                                                                                                              \
-        if (vec) rms_fused_kernel<WT, THREADS, EPT, true><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);   \
-        else rms_fused_kernel<WT, THREADS, EPT, false><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);      \
+#define ZK_RMS_LAUNCH(THREADS, EPT, WPE)                                                                                   \
+    do {                                                                                                                   \
+        if (vec) rms_fused_kernel<WT, THREADS, EPT, true, WPE><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);   \
+        else rms_fused_kernel<WT, THREADS, EPT, false, WPE><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);      \
     } while (0)
-    if (N <= 512) ZK_RMS_LAUNCH(256, 2);
-    else if (N <= 2048) ZK_RMS_LAUNCH(256, 8);
-    else if (N <= 4096) ZK_RMS_LAUNCH(512, 8);
-    else if (N <= 8192) ZK_RMS_LAUNCH(ZK_RMS_T8K, ZK_RMS_E8K);
-    else if (N <= 16384) ZK_RMS_LAUNCH(1024, 16);
+    if (N <= 512) ZK_RMS_LAUNCH(256, 2, 1);
+    else if (N <= 2048) ZK_RMS_LAUNCH(256, 8, 1);
+    else if (N <= 4096) ZK_RMS_LAUNCH(512, 8, 1);
+    else if (N <= 8192) ZK_RMS_LAUNCH(512, 16, 6);
+    else if (N <= 16384) ZK_RMS_LAUNCH(1024, 16, 1);
     else {
         rms_stat_kernel<<<grid, dim3(kRmsThreads), 0, 0>>>(A, rms, N, eps, dim);
         if (check_launch(name)) launch_apply<WT>(name, A, W, rms, C, M, N);
