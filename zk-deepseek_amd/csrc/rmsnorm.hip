@@ -247,6 +247,8 @@ __device__ __forceinline__ U192 block_sum_u192(U192 acc, U192 *red)
     return tot;
 }
 
+typedef int v4i_r __attribute__((ext_vector_type(4)));
+
 // Statistic only: one workgroup per row, any N.
 __global__ __launch_bounds__(kRmsThreads) void rms_stat_kernel(const int64_t *__restrict__ A, int64_t *__restrict__ rms,
                                                                int N, int64_t eps, int64_t dim)
@@ -254,12 +256,32 @@ __global__ __launch_bounds__(kRmsThreads) void rms_stat_kernel(const int64_t *__
     __shared__ U192 red[kRmsThreads / 64];
     const int64_t *a = A + (long)blockIdx.x * N;
     SquareSum sq;
-    for (int i = threadIdx.x; i < N; i += kRmsThreads) sq.add(a[i]);
+    if (N % 2 == 0 && ((uintptr_t)A & 15) == 0) {
+        // two elements per load, four loads in flight per thread
+        const int pairs = N / 2;
+        int i = threadIdx.x;
+        for (; i + 3 * kRmsThreads < pairs; i += 4 * kRmsThreads) {
+            v4i_r t[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                t[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a) + i + u * kRmsThreads);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                sq.add((int64_t)(((uint64_t)(uint32_t)t[u][1] << 32) | (uint32_t)t[u][0]));
+                sq.add((int64_t)(((uint64_t)(uint32_t)t[u][3] << 32) | (uint32_t)t[u][2]));
+            }
+        }
+        for (; i < pairs; i += kRmsThreads) {
+            const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a) + i);
+            sq.add((int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]));
+            sq.add((int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]));
+        }
+    } else {
+        for (int i = threadIdx.x; i < N; i += kRmsThreads) sq.add(a[i]);
+    }
     U192 tot = block_sum_u192<kRmsThreads>(sq.total(), red);
     if (threadIdx.x == 0) rms[blockIdx.x] = rms_finalize(tot, eps, dim);
 }
-
-typedef int v4i_r __attribute__((ext_vector_type(4)));
 
 // Normalisation only, rms given (the reference's rms_norm_32 / rms_norm_64 contract).  A workgroup covers
 // 256 * kApplyEpt consecutive elements of one row; VEC: N is even and the rows are 16-byte aligned.
