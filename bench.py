@@ -211,6 +211,22 @@ def main():
             hbm("rmsnorm_fused_%dx7168" % Mr,
                 lambda: K.lib.rms_norm_fused_32(Ar.data_ptr(), Wr.data_ptr(), rr.data_ptr(), Cr.data_ptr(), Mr, 7168, 1, 7168),
                 Ar.numel(), extra_bytes=4.0 * 7168 + 8.0 * Mr, steps=20)
+            if Mr == 16384:
+                # the residual connection in front of the norm, fused (32 B/element) against torch's multiply and add
+                # followed by the fused norm (model.py:1465-1468)
+                Yr = randint(g6, -(1 << 25), 1 << 25, (Mr, 7168)).cuda()
+                Xo = torch.empty_like(Ar)
+                nm = "rmsnorm_residual_fused_%dx7168_32B_per_element" % Mr
+                hbm(nm, lambda: K.lib.rms_norm_residual_fused_32(Ar.data_ptr(), Yr.data_ptr(), 12, Wr.data_ptr(), Xo.data_ptr(),
+                                                                 rr.data_ptr(), Cr.data_ptr(), Mr, 7168, 1, 7168),
+                    Ar.numel(), bytes_per_elem=32.0, steps=20)
+
+                def chain0():
+                    xn = Ar + Yr * (1 << 12)
+                    K.lib.rms_norm_fused_32(xn.data_ptr(), Wr.data_ptr(), rr.data_ptr(), Cr.data_ptr(), Mr, 7168, 1, 7168)
+
+                extra[nm]["unfused_chain_ms"] = timed(K, chain0, 5, 2)
+                del Yr, Xo
             del Ar, Cr
 
         # the two fusions against the chains they replace (the reference's tensor ops around the kernel, on torch)

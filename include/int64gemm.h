@@ -111,6 +111,15 @@ void rms_norm_fused_32(const int64_t *A, const int32_t *W, int64_t *rms, int64_t
 void rms_norm_fused_64(const int64_t *A, const int64_t *W, int64_t *rms, int64_t *C,
                        int M, int N, int64_t eps, int64_t dim);
 
+/* The residual connection fused into the norm behind it: X' = X + Y * 2^k (wrapping int64, as the tensor ops of
+ * inference/model.py:1465 and :1472 compute it) is stored to Xout [M,N] (which may be X itself) and normalised in
+ * the same pass over the row: C = floor(X' * W / rms), rms as above.  32 bytes per element instead of the 56 of
+ * multiply, add and norm as three tensor ops.  0 <= k <= 63. */
+void rms_norm_residual_fused_32(const int64_t *X, const int64_t *Y, int k, const int32_t *W, int64_t *Xout, int64_t *rms,
+                                int64_t *C, int M, int N, int64_t eps, int64_t dim);
+void rms_norm_residual_fused_64(const int64_t *X, const int64_t *Y, int k, const int64_t *W, int64_t *Xout, int64_t *rms,
+                                int64_t *C, int M, int N, int64_t eps, int64_t dim);
+
 /* 1: softmax_q19/q21 also overwrite R with the per-element weights, as the reference's kernels do
  * (inference/int64_gemm.cu:708,729 and :629,650).  0 (default): R is left untouched. */
 void zk_softmax_clobber_input(int on);

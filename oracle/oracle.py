@@ -170,6 +170,14 @@ def RMS_Norm_int64(A, W, eps, dim):
     return rms_norm_apply(A, W, rms), rms
 
 
+def RMS_Norm_residual_int64(X, Y, k, W, eps, dim):
+    """(X', C, rms) for X' = X + Y * 2^k in wrapping int64 (torch's tensor ops at inference/model.py:1465, 1472)
+    followed by the norm of inference/model.py:1468 / the next block's :1453."""
+    Xn = (_c(X).view(np.uint64) + (_c(Y).view(np.uint64) << np.uint64(k))).view(np.int64)
+    C, rms = RMS_Norm_int64(Xn, W, eps, dim)
+    return Xn, C, rms
+
+
 def _lut(fn):
     lut = np.zeros((256,), np.int64)
     fn(_p(lut))

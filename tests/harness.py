@@ -32,6 +32,11 @@ class CpuBackend:
     def rmsnorm(self, x2d, w, dim):
         return self.o.RMS_Norm_int64(x2d, w, 1, dim)[0]
 
+    def residual_rmsnorm(self, x2d, y2d, k, w, dim):
+        """(x + y * 2^k, its norm): inference/model.py:1465-1468 op by op"""
+        x2d = x2d + y2d * (1 << k)
+        return x2d, self.rmsnorm(x2d, w, dim)
+
     def softmax_scores(self, s1, s2, mask):
         """(scores, probabilities): inference/model.py:896-915 as the reference writes it, op by op"""
         scores = (s1 + s2) * 94 // 695           # floor division (model.py:897)
@@ -98,6 +103,7 @@ class GpuBackend:
 
     softmax_scores = CpuBackend.softmax_scores   # the same op-by-op chain, on torch tensors
     silu_mul = CpuBackend.silu_mul
+    residual_rmsnorm = CpuBackend.residual_rmsnorm
 
     def rope(self, x, table):
         return self.k.complex_int64_mul_broadcast(x.contiguous(), table.contiguous())
@@ -134,6 +140,10 @@ class FusedGpuBackend(GpuBackend):
         out = self.t.empty_like(r1)
         self.k.silu_mul_q23(r1.contiguous(), r2.contiguous(), out)
         return out
+
+    def residual_rmsnorm(self, x2d, y2d, k, w, dim):
+        xn, c, _ = self.k.RMS_Norm_residual_int64(x2d.contiguous(), y2d.contiguous(), k, w, 1, dim)
+        return xn, c
 
     def route(self, scores, bias_host, cfg):
         bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
@@ -332,7 +342,7 @@ def moe(be, x, P, cfg):
 def decoder_layer(be, x, P, freqs, cfg):
     """Block.forward for a MoE layer (inference/model.py:1430-1475): x Q31 residual stream [1,S,dim]"""
     a = be.rmsnorm(x[0], P["attn_norm"], cfg["dim"])[None]
-    x = x + mla(be, a, P, freqs, cfg) * (1 << 12)               # model.py:1465
-    f = be.rmsnorm(x[0], P["ffn_norm"], cfg["dim"])[None]
+    x, f = be.residual_rmsnorm(x[0], mla(be, a, P, freqs, cfg)[0], 12, P["ffn_norm"], cfg["dim"])   # model.py:1465-1468
+    x, f = x[None], f[None]
     y, idx = moe(be, f, P, cfg)
     return x + y * (1 << 8), idx                                 # model.py:1472

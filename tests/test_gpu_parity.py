@@ -456,6 +456,55 @@ def test_rmsnorm_quotients_next_to_integers(K, oracle, r, w32):
         assert np.array_equal(host(C), oracle.rms_norm_apply(np.ascontiguousarray(A), W, rms))
 
 
+@pytest.mark.parametrize("N", [7, 512, 1536, 4096, 7168, 9001, 20000])
+@pytest.mark.parametrize("k,w32,inplace", [(12, True, False), (8, False, True), (0, True, True), (63, False, False)])
+def test_rmsnorm_residual_fusion(K, oracle, N, k, w32, inplace):
+    """x + y * 2^k (wrapping) stored and normalised in one pass (model.py:1465-1468): every row-length tier, odd and
+    even N, in place or not, sums that wrap around 2^64"""
+    rng = np.random.default_rng(N + k)
+    M = 5
+    X = rand_i64(rng, (M, N), 37)
+    Y = rand_i64(rng, (M, N), 40 if k < 20 else 63)
+    if k == 8:
+        X[1, :5] = [(1 << 63) - 1, -(1 << 63), (1 << 62), -1, 0]          # the sum wraps
+        Y[1, :5] = [(1 << 54), -(1 << 54) - 1, (1 << 55) - 1, 1, 0]
+    W = rng.integers(1 << 5, 1 << 20, size=(N,), dtype=np.int32) if w32 else rand_i64(rng, (N,), 40)
+    Xd = dev(X)
+    Xn, C, rms = K.RMS_Norm_residual_int64(Xd, dev(Y), k, dev(W), 1, N, inplace=inplace)
+    Xe, Ce, rmse = oracle.RMS_Norm_residual_int64(X, Y, k, W, 1, N)
+    assert (Xn.data_ptr() == Xd.data_ptr()) == inplace
+    assert np.array_equal(host(Xn), Xe)
+    assert np.array_equal(rms[:M].numpy(), rmse)
+    assert np.array_equal(host(C), Ce)
+
+
+def test_rmsnorm_residual_fusion_unaligned_and_bad_arguments(K, oracle):
+    rng = np.random.default_rng(77)
+    M, N = 3, 1000
+    X, Y = rand_i64(rng, (M, N), 37), rand_i64(rng, (M, N), 30)
+    W = rng.integers(1, 1 << 20, size=(N,), dtype=np.int32)
+    # rows that start 8 bytes off a 16-byte boundary take the element-wise path
+    buf = torch.zeros((M * N + 1,), dtype=torch.int64, device="cuda")
+    Xd = buf[1:].view(M, N)
+    Xd.copy_(dev(X))
+    Yd, Wd = dev(Y), dev(W)
+    Xo = torch.empty((M, N), dtype=torch.int64, device="cuda")
+    C = torch.empty((M, N), dtype=torch.int64, device="cuda")
+    r = torch.empty((M,), dtype=torch.int64, device="cuda")
+    K.lib.rms_norm_residual_fused_32(Xd.data_ptr(), Yd.data_ptr(), 12, Wd.data_ptr(), Xo.data_ptr(), r.data_ptr(), C.data_ptr(), M, N, 1, N)
+    torch.cuda.synchronize()
+    K._check("residual norm")
+    Xe, Ce, rmse = oracle.RMS_Norm_residual_int64(X, Y, 12, W, 1, N)
+    assert np.array_equal(host(Xo), Xe) and np.array_equal(host(C), Ce) and np.array_equal(host(r), rmse)
+    for bad_k in (-1, 64):
+        K.lib.rms_norm_residual_fused_32(Xd.data_ptr(), Yd.data_ptr(), bad_k, Wd.data_ptr(), Xo.data_ptr(), r.data_ptr(), C.data_ptr(), M, N, 1, N)
+        assert K.lib.zk_last_error() == 1
+        K.lib.zk_clear_error()
+    K.lib.rms_norm_residual_fused_32(Xd.data_ptr(), None, 12, Wd.data_ptr(), Xo.data_ptr(), r.data_ptr(), C.data_ptr(), M, N, 1, N)
+    assert K.lib.zk_last_error() == 1
+    K.lib.zk_clear_error()
+
+
 def test_rmsnorm_model_shape(K, oracle):
     """[256,7168] at residual-stream magnitudes (|x| up to ~2^37, Q31) with int32 Q21 weights"""
     g = torch.Generator(device="cpu").manual_seed(600)

@@ -353,10 +353,14 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
 // WPE: waves per SIMD the register allocation must leave room for.  Rows of 4K-8K elements run three workgroups of
 // eight waves per compute unit (WPE 6, 80 registers): measured, a third row in flight is worth more than the few
 // registers spilled for it, a fourth is not.
-template <typename WT, int THREADS, int EPT, bool VEC, int WPE>
-__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) void rms_fused_kernel(const int64_t *__restrict__ A, const WT *__restrict__ W,
+// RES: the row that is normalised is A + Y * 2^k (wrapping int64 arithmetic, as the tensor ops of the reference's
+// residual connection, inference/model.py:1465, 1472), and that sum is also stored to Xout (which may be A itself).
+struct RmsResidual { const int64_t *Y; int64_t *Xout; int k; };
+
+template <typename WT, int THREADS, int EPT, bool VEC, int WPE, bool RES>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) void rms_fused_kernel(const int64_t *A, const WT *__restrict__ W,
                                                                 int64_t *__restrict__ rms, int64_t *__restrict__ C,
-                                                                int N, int64_t eps, int64_t dim)
+                                                                int N, int64_t eps, int64_t dim, RmsResidual res)
 {
     __shared__ U192 red[THREADS / 64];
     __shared__ int64_t rms_s;
@@ -375,6 +379,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
                 wp[j] = load_w_pair(W, i, w_vec);
                 v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
                 v[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
+                if (RES) {
+                    const v4i_r u = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(res.Y + row * N + i));
+                    const uint64_t y0 = ((uint64_t)(uint32_t)u[1] << 32) | (uint32_t)u[0];
+                    const uint64_t y1 = ((uint64_t)(uint32_t)u[3] << 32) | (uint32_t)u[2];
+                    v[2 * j] = (int64_t)((uint64_t)v[2 * j] + (y0 << res.k));
+                    v[2 * j + 1] = (int64_t)((uint64_t)v[2 * j + 1] + (y1 << res.k));
+                    const v4i_r o = { (int)(uint32_t)v[2 * j], (int)(uint32_t)((uint64_t)v[2 * j] >> 32),
+                                      (int)(uint32_t)v[2 * j + 1], (int)(uint32_t)((uint64_t)v[2 * j + 1] >> 32) };
+                    *reinterpret_cast<v4i_r *>(res.Xout + row * N + i) = o;
+                }
                 sq.add(v[2 * j]);
                 sq.add(v[2 * j + 1]);
             }
@@ -383,7 +397,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
             const int i = j * THREADS + threadIdx.x;
-            if (i < N) { v[j] = a[i]; sq.add(v[j]); }
+            if (i < N) {
+                v[j] = a[i];
+                if (RES) {
+                    v[j] = (int64_t)((uint64_t)v[j] + ((uint64_t)res.Y[row * N + i] << res.k));
+                    res.Xout[row * N + i] = v[j];
+                }
+                sq.add(v[j]);
+            }
         }
     }
     U192 tot = block_sum_u192<THREADS>(sq.total(), red);
@@ -457,17 +478,35 @@ static bool stat_args_ok(const char *name, int64_t eps, int64_t dim)
     return true;
 }
 
+// Y * 2^k added to A, element by element (only for rows too long for the fused kernel)
+__global__ __launch_bounds__(256) void residual_add_kernel(const int64_t *A, const int64_t *__restrict__ Y, int64_t *Xout, long n, int k)
+{
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+        Xout[i] = (int64_t)((uint64_t)A[i] + ((uint64_t)Y[i] << k));
+}
+
 template <typename WT>
 static void launch_fused(const char *name, const int64_t *A, const WT *W, int64_t *rms, int64_t *C, int M, int N,
-                         int64_t eps, int64_t dim)
+                         int64_t eps, int64_t dim, const RmsResidual *res = nullptr)
 {
     if (!rms_args_ok(name, A, W, rms, C, M, N) || !stat_args_ok(name, eps, dim)) return;
-    const bool vec = N % 2 == 0 && (((uintptr_t)A | (uintptr_t)C) & 15) == 0;
+    if (!W) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    uintptr_t align = (uintptr_t)A | (uintptr_t)C;
+    RmsResidual r = { nullptr, nullptr, 0 };
+    if (res) {
+        if (!res->Y || !res->Xout) { set_error(kBadArgument, "%s: null pointer", name); return; }
+        if (res->k < 0 || res->k > 63) { set_error(kBadArgument, "%s: shift %d outside 0..63", name, res->k); return; }
+        r = *res;
+        align |= (uintptr_t)r.Y | (uintptr_t)r.Xout;
+    }
+    const bool vec = N % 2 == 0 && (align & 15) == 0;
     const dim3 grid((unsigned)M);
-#define ZK_RMS_LAUNCH(THREADS, EPT, WPE)                                                                                   \
-    do {                                                                                                                   \
-        if (vec) rms_fused_kernel<WT, THREADS, EPT, true, WPE><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);   \
-        else rms_fused_kernel<WT, THREADS, EPT, false, WPE><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim);      \
+#define ZK_RMS_LAUNCH2(THREADS, EPT, WPE, VEC, RES) \
+    rms_fused_kernel<WT, THREADS, EPT, VEC, WPE, RES><<<grid, dim3(THREADS), 0, 0>>>(A, W, rms, C, N, eps, dim, r)
+#define ZK_RMS_LAUNCH(THREADS, EPT, WPE)                                                   \
+    do {                                                                                   \
+        if (res) { if (vec) ZK_RMS_LAUNCH2(THREADS, EPT, WPE, true, true); else ZK_RMS_LAUNCH2(THREADS, EPT, WPE, false, true); }    \
+        else { if (vec) ZK_RMS_LAUNCH2(THREADS, EPT, WPE, true, false); else ZK_RMS_LAUNCH2(THREADS, EPT, WPE, false, false); }      \
     } while (0)
     if (N <= 512) ZK_RMS_LAUNCH(256, 2, 1);
     else if (N <= 2048) ZK_RMS_LAUNCH(256, 8, 1);
@@ -475,11 +514,19 @@ static void launch_fused(const char *name, const int64_t *A, const WT *W, int64_
     else if (N <= 8192) ZK_RMS_LAUNCH(512, 16, 6);
     else if (N <= 16384) ZK_RMS_LAUNCH(1024, 16, 1);
     else {
-        rms_stat_kernel<<<grid, dim3(kRmsThreads), 0, 0>>>(A, rms, N, eps, dim);
-        if (check_launch(name)) launch_apply<WT>(name, A, W, rms, C, M, N);
+        const int64_t *src = A;
+        if (res) {
+            const long n = (long)M * N;
+            residual_add_kernel<<<dim3((unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536)), dim3(256), 0, 0>>>(A, r.Y, r.Xout, n, r.k);
+            if (!check_launch(name)) return;
+            src = r.Xout;
+        }
+        rms_stat_kernel<<<grid, dim3(kRmsThreads), 0, 0>>>(src, rms, N, eps, dim);
+        if (check_launch(name)) launch_apply<WT>(name, src, W, rms, C, M, N);
         return;
     }
 #undef ZK_RMS_LAUNCH
+#undef ZK_RMS_LAUNCH2
     check_launch(name);
 }
 
@@ -515,6 +562,20 @@ void rms_norm_fused_64(const int64_t *A, const int64_t *W, int64_t *rms, int64_t
                        int64_t dim)
 {
     zk::launch_fused<int64_t>("rms_norm_fused_64", A, W, rms, C, M, N, eps, dim);
+}
+
+void rms_norm_residual_fused_32(const int64_t *X, const int64_t *Y, int k, const int32_t *W, int64_t *Xout, int64_t *rms,
+                                int64_t *C, int M, int N, int64_t eps, int64_t dim)
+{
+    const zk::RmsResidual res = { Y, Xout, k };
+    zk::launch_fused<int32_t>("rms_norm_residual_fused_32", X, W, rms, C, M, N, eps, dim, &res);
+}
+
+void rms_norm_residual_fused_64(const int64_t *X, const int64_t *Y, int k, const int64_t *W, int64_t *Xout, int64_t *rms,
+                                int64_t *C, int M, int N, int64_t eps, int64_t dim)
+{
+    const zk::RmsResidual res = { Y, Xout, k };
+    zk::launch_fused<int64_t>("rms_norm_residual_fused_64", X, W, rms, C, M, N, eps, dim, &res);
 }
 
 }  // extern "C"

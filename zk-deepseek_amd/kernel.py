@@ -58,6 +58,8 @@ lib.wkv_b_bf16_to_int32.argtypes = [_vp, _vp, _ci, _ci]
 lib.rms_stat_int64.argtypes = [_vp, _vp, _ci, _ci, _ll, _ll]
 lib.rms_norm_fused_32.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
 lib.rms_norm_fused_64.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
+lib.rms_norm_residual_fused_32.argtypes = [_vp, _vp, _ci, _vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
+lib.rms_norm_residual_fused_64.argtypes = [_vp, _vp, _ci, _vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
 lib.zk_last_error.restype = _ci
 lib.zk_last_error_string.restype = ctypes.c_char_p
 lib.zk_softmax_clobber_input.argtypes = [_ci]
@@ -233,6 +235,28 @@ def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim):
     _check("RMS_Norm_int64")
     rms[:M] = rms_gpu[:M].cpu()
     return (C, rms)
+
+
+def RMS_Norm_residual_int64(X: torch.Tensor, Y: torch.Tensor, k: int, W: torch.Tensor, eps, dim, inplace=False):
+    """The residual connection and the norm behind it in one pass over the row (inference/model.py:1465-1468,
+    1472 with the next block's :1453): X' = X + Y * 2^k in wrapping int64, C = RMSNorm(X') with weights W.
+    Returns (X', C, rms buffer); inplace=True writes X' over X."""
+    global rms, rms_gpu
+    assert X.dtype == torch.int64 and Y.dtype == torch.int64 and X.shape == Y.shape
+    assert X.is_cuda and Y.is_cuda and W.is_cuda and X.is_contiguous() and Y.is_contiguous()
+    assert X.ndim == 2
+    M, N = X.shape
+    assert M <= rms.shape[0], "the rms buffer holds 500 rows, as in the reference"
+    if rms_gpu is None or rms_gpu.device != X.device:
+        rms_gpu = torch.zeros((500,), dtype=torch.int64, device=X.device)
+    Xout = X if inplace else torch.empty_like(X)
+    C = torch.empty((M, N), dtype=torch.int64, device=X.device)
+    assert W.dtype in (torch.int32, torch.int64)
+    fn = lib.rms_norm_residual_fused_32 if W.dtype == torch.int32 else lib.rms_norm_residual_fused_64
+    fn(X.data_ptr(), Y.data_ptr(), k, W.data_ptr(), Xout.data_ptr(), rms_gpu.data_ptr(), C.data_ptr(), M, N, eps, dim)
+    _check("RMS_Norm_residual_int64")
+    rms[:M] = rms_gpu[:M].cpu()
+    return (Xout, C, rms)
 
 
 atexit.register(lambda: lib.zk_dump_flush())
