@@ -321,6 +321,35 @@ def main():
         finally:
             shutil.rmtree(tmpd, ignore_errors=True)
 
+        # the four MLA einsums at config 3's shape (S = T = 1024, 128 heads, absorb mode: model.py:884-936), Q30
+        # activations against Q24 cache entries / int32 Q25 weights
+        ge = torch.Generator(device="cuda").manual_seed(900)
+        rnd = lambda bits, *shape: torch.randint(-(1 << bits), 1 << bits, shape, generator=ge, dtype=torch.int64, device="cuda")
+
+        def einsum_leg(name, fn, macs):
+            ms = timed(K, fn, 5, 2)
+            K._check(name)
+            _p, la, lb = K.gemm_last_plan()
+            extra[name] = {"ms": ms, "gmacs": macs / ms / 1e6, "macs": macs, "limbs_a": la, "limbs_b": lb,
+                           "digit_pairs": K.gemm_last_pairs()}
+
+        Se, He, Ce, De, Re = 1024, 128, 512, 128, 64
+        qn, wb1 = rnd(30, 1, Se, He, De), rnd(25, He, De, Ce).to(torch.int32)
+        einsum_leg("einsum_bshd_hdc_bshc_1x1024x128x128_to_512", lambda: K.einsum_bshd_hdc_bshc(qn, wb1, 21), Se * He * De * Ce)
+        del qn, wb1
+        qa, kvc = rnd(30, 1, Se, He, Ce), rnd(24, 1, Se, Ce)
+        einsum_leg("einsum_bshc_btc_bsht_1x1024x128x512_T1024", lambda: K.einsum_bshc_btc_bsht(qa, kvc, 23), Se * He * Se * Ce)
+        del qa
+        qp, pec = rnd(30, 1, Se, He, Re), rnd(24, 1, Se, Re)
+        einsum_leg("einsum_bshc_btc_bsht_1x1024x128x64_T1024", lambda: K.einsum_bshc_btc_bsht(qp, pec, 21), Se * He * Se * Re)
+        del qp, pec
+        pp = torch.randint(0, 1 << 19, (1, Se, He, Se), generator=ge, dtype=torch.int64, device="cuda")
+        einsum_leg("einsum_bsht_btc_bshc_1x1024x128xT1024_to_512", lambda: K.einsum_bsht_btc_bshc(pp, kvc, 23), Se * He * Se * Ce)
+        del pp, kvc
+        oo, wb2 = rnd(30, 1, Se, He, Ce), rnd(25, He, De, Ce).to(torch.int32)
+        einsum_leg("einsum_bshc_hdc_bshd_1x1024x128x512_to_128", lambda: K.einsum_bshc_hdc_bshd(oo, wb2, 21), Se * He * De * Ce)
+        del oo, wb2
+
         # RoPE and the float -> fixed converters (weight-loading path), by their own algorithmic bytes per element
         gq = torch.Generator(device="cpu").manual_seed(700)
         q_pe = randint(gq, -(1 << 30), 1 << 30, (1, 4096, 128, 32, 2)).cuda()

@@ -31,7 +31,8 @@ extern "C" {
 /* C[b,m,n] = (sum_k (A[b,m,k]/a_rescale) * (B[n,k]/b_rescale)) >> c_rescale, 128-bit wrapping sum,
  * `/` truncates toward zero; R = sum mod 2^c_rescale.  A [Bdim,M,K] i64, B [N,K], C,R [Bdim,M,N] i64.
  * Replaces inference/int64_gemm.cu:79-90 (B int64) and :36-47 (B int32); bound at inference/kernel.py:209-225.
- * c_rescale must be in [0,63]; the rescales must be non-zero. */
+ * c_rescale must be in [0,63]; the rescales must be non-zero.  R may be NULL (the reference always stores it, but
+ * only three of the model's callers read it): then no remainder is stored. */
 void int64_64_bmm_broadcast_launcher(const int64_t *A, const int64_t *B, int64_t *C, int64_t *R,
                                      const int64_t a_rescale, const int64_t b_rescale, const int64_t c_rescale,
                                      int Bdim, int M, int K, int N);

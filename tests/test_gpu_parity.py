@@ -117,6 +117,21 @@ def test_gemm_few_rows_many_columns(K, oracle, shape, bits):
 
 
 @pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("shape", [(1, 70, 300, 150), (2, 8, 2048, 512), (1, 300, 1024, 300)])
+def test_gemm_without_remainder(K, oracle, path, shape):
+    """R = NULL: the quotient is the same and nothing is stored for the remainder (whole tiles, split-K tiles and
+    the vector-ALU kernel each have their own epilogue)"""
+    Bd, M, Kd, N = shape
+    rng = np.random.default_rng(sum(shape))
+    A, W = rand_i64(rng, (Bd, M, Kd), 37), rand_i32(rng, (N, Kd), 31)
+    K.lib.zk_gemm_set_path(path)
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 29, want_remainder=False)
+    assert R is None
+    assert np.array_equal(host(C), oracle.int64_bmm_broadcast(A, W, 1, 1, 29)[0])
+    K.lib.zk_gemm_set_path(0)
+
+
+@pytest.mark.parametrize("path", PATHS)
 def test_gemm_operand_divisors(K, oracle, path):
     """head projection divides the weights by 256 (inference/model.py:1519); division truncates toward zero"""
     rng = np.random.default_rng(5)

@@ -116,8 +116,9 @@ def fp8_gemm(*args, **kwargs):
     raise NotImplementedError("fp8_gemm belongs to the fp8 path, which the int64 model never reaches")
 
 
-def int64_bmm_broadcast(A: torch.Tensor, B: torch.Tensor, a_rescale, b_rescale, c_rescale):
-    """(B, M, K) x (N, K) -> quotient C and remainder R, both (B, M, N) int64."""
+def int64_bmm_broadcast(A: torch.Tensor, B: torch.Tensor, a_rescale, b_rescale, c_rescale, want_remainder=True):
+    """(B, M, K) x (N, K) -> quotient C and remainder R, both (B, M, N) int64.
+    want_remainder=False (not in the reference) skips the remainder's store and returns (C, None)."""
     assert A.dtype == torch.int64
     assert A.is_cuda and B.is_cuda
     Bdim, M, K = A.shape
@@ -125,13 +126,14 @@ def int64_bmm_broadcast(A: torch.Tensor, B: torch.Tensor, a_rescale, b_rescale, 
     assert K2 == K
 
     C = torch.empty((Bdim, M, N), dtype=torch.int64, device=A.device)
-    R = torch.empty((Bdim, M, N), dtype=torch.int64, device=A.device)
+    R = torch.empty((Bdim, M, N), dtype=torch.int64, device=A.device) if want_remainder else None
+    r_ptr = R.data_ptr() if want_remainder else None
 
     if B.dtype == torch.int64:
-        lib.int64_64_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), R.data_ptr(),
+        lib.int64_64_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), r_ptr,
                                             a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
     elif B.dtype == torch.int32:
-        lib.int64_32_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), R.data_ptr(),
+        lib.int64_32_bmm_broadcast_launcher(A.data_ptr(), B.data_ptr(), C.data_ptr(), r_ptr,
                                             a_rescale, b_rescale, c_rescale, Bdim, M, K, N)
     else:
         raise TypeError(f"Unsupported B type: {B.dtype}")
