@@ -27,8 +27,8 @@ I8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20, help="untimed calls before the timed steps (at least; see SPIN_UP_MS)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,cpu,calib (default gemm,extra,cpu)")
     return ap.parse_args()
@@ -46,12 +46,30 @@ def full_range(gen, shape):
     return (hi << 32) | lo
 
 
+SPIN_UP_MS = 60.0    # an idle device needs some 40 ms of work to reach its clocks (measured: the first 50 config-4
+                     # GEMM calls after a pause average 0.76 ms, every later 50 average 0.70 ms)
+
+
+def spin_up(fn, at_least=0):
+    """untimed calls of fn: `at_least` of them, and as many more as it takes to keep the device busy for SPIN_UP_MS"""
+    import torch
+    calls = at_least
+    for _ in range(at_least):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SPIN_UP_MS:
+        for _ in range(4):
+            fn()
+        calls += 4
+        torch.cuda.synchronize()
+    return calls
+
+
 def timed(K, fn, steps, warmup):
     """average milliseconds per call, measured with HIP events on the null stream (where the library launches)"""
     import torch
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
+    spin_up(fn, warmup)
     K.lib.zk_timer_start()
     for _ in range(steps):
         fn()
@@ -107,9 +125,7 @@ def main():
         K.lib.int64_64_bmm_broadcast_launcher(A.data_ptr(), W.data_ptr(), Cb.data_ptr(), Rb.data_ptr(),
                                               1, 1, c, 1, M, Kd, N)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    warmup_calls = spin_up(step, args.warmup)
     t0 = time.perf_counter()
     K.lib.zk_timer_start()
     for _ in range(args.steps):
@@ -385,7 +401,7 @@ def main():
 
     out = {
         "metric": "int64 GEMM Gmac/s @7168x576 & 18432x7168 + softmax/SiLU HBM GB/s, 1 MI355X",
-        "value": value, "unit": "Gmac/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": value, "unit": "Gmac/s", "n_gpus": 1, "steps": args.steps, "warmup": warmup_calls,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int64", "data": "synthetic",
         "config": {"workload": "config4: int64 GEMM Y[512,18432] = X[512,7168] @ W[18432,7168]^T, int64 W, "
