@@ -374,6 +374,13 @@ def main():
         hbm("rope_1x4096x128x64", lambda: K.lib.complex_int64_mul(q_pe.data_ptr(), tab.data_ptr(), out.data_ptr(), 1, 4096, 128, 32),
             q_pe.numel(), steps=20)
         del q_pe, out
+        # checkpoint quantisation (convert2.py): block-scaled fp8 weights -> int32, 1 byte read + 4 written per weight
+        w8 = torch.randint(0, 256, (18432, 7168), generator=gq, dtype=torch.uint8).cuda()
+        s8 = (torch.rand((144, 56), generator=gq, dtype=torch.float32) * 1e-3 + 1e-5).cuda()
+        o8 = torch.empty((18432, 7168), dtype=torch.int32, device="cuda")
+        hbm("fp8_block_scaled_to_int32_18432x7168", lambda: K.lib.fp8_block_scaled_to_int32(w8.data_ptr(), s8.data_ptr(), o8.data_ptr(), 18432, 7168, 30),
+            w8.numel(), bytes_per_elem=5.0, steps=20)
+        del w8, o8
         wb = torch.randn((18432, 7168), generator=gq, dtype=torch.float32)
         w16 = wb.to(torch.bfloat16).cuda()
         o32 = torch.empty((18432, 7168), dtype=torch.int32, device="cuda")

@@ -214,6 +214,18 @@ double zk_probe_mfma_i8_tops(int with_lds, int random_data, int steps);
 void zk_timer_start(void);
 float zk_timer_stop_ms(void);   /* records the stop event, waits for it, returns elapsed milliseconds */
 
+/* Float checkpoint -> fixed-point weights, the quantisation of inference/convert2.py on the device.
+ * fp8_block_scaled_to_int32: out = (weight_dequant(w, scale).to(float32) * 2^k).round().to(int32)
+ * (convert2.py:144-147, 308-311 and the like; weight_dequant is the Triton kernel of inference/kernel.py:67-117):
+ * w [rows,cols] OCP e4m3fn bytes, scale [ceil(rows/128), ceil(cols/128)] float32, one scale per 128x128 block; the
+ * product is rounded to bfloat16 (the reference's default dtype, convert2.py:185) before it is scaled by 2^k, rounded
+ * half to even and converted as the reference's device converts (saturating, NaN -> 0).  0 <= k <= 127.
+ * bf16_scaled_round_to_int32/64: out = (p.to(float32) * 2^k).round().to(int32|int64) for n bfloat16 values
+ * (convert2.py:250-262, 290-295, 353-359). */
+void fp8_block_scaled_to_int32(const uint8_t *w, const float *scale, int32_t *out, int rows, int cols, int k);
+void bf16_scaled_round_to_int32(const uint16_t *in, int32_t *out, long n, int k);
+void bf16_scaled_round_to_int64(const uint16_t *in, int64_t *out, long n, int k);
+
 #ifdef __cplusplus
 }
 #endif

@@ -335,6 +335,64 @@ def wkv_b_bf16_to_int32(bits):
     return out
 
 
+def _e4m3fn_table():
+    """the 256 values of an OCP e4m3fn byte as float32: 1 sign, 4 exponent (bias 7), 3 mantissa bits; no infinities,
+    S.1111.111 is NaN"""
+    t = np.empty(256, np.float32)
+    for b in range(256):
+        e, m = (b >> 3) & 15, b & 7
+        if e == 15 and m == 7:
+            v = float("nan")
+        elif e == 0:
+            v = m * 2.0 ** -9
+        else:
+            v = (1 + m / 8.0) * 2.0 ** (e - 7)
+        t[b] = -v if b & 0x80 else v
+    return t
+
+
+def _round_to_bf16(x):
+    """float32 array -> nearest bfloat16 (ties to even), returned as float32"""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    r = np.where(np.isnan(x), np.uint32(0x7FC00000), r).astype(np.uint32)
+    return r.view(np.float32)
+
+
+def _round_to_int(z, dtype):
+    """round half to even, then the float -> integer conversion of the reference's device: saturating, NaN -> 0"""
+    info = np.iinfo(dtype)
+    r = np.rint(z.astype(np.float64))
+    out = np.zeros(z.shape, dtype)
+    ok = ~np.isnan(r)
+    hi, lo = r >= float(info.max) + 1.0, r <= float(info.min)
+    mid = ok & ~hi & ~lo
+    out[mid] = r[mid].astype(dtype)
+    out[ok & hi] = info.max
+    out[ok & lo] = info.min
+    return out
+
+
+def fp8_block_scaled_to_int32(w_bytes, scale, k, block=128):
+    """(weight_dequant(w, scale).to(float32) * 2**k).round().to(int32): inference/convert2.py:144-147 with the Triton
+    kernel of inference/kernel.py:67-117 (x.to(float32) * s, stored as bfloat16) restated operation by operation."""
+    w_bytes = np.ascontiguousarray(w_bytes, np.uint8)
+    rows, cols = w_bytes.shape
+    s = np.repeat(np.repeat(np.ascontiguousarray(scale, np.float32), block, axis=0), block, axis=1)[:rows, :cols]
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = _round_to_bf16(_e4m3fn_table()[w_bytes] * s)             # float32 multiply, then bfloat16 store
+        z = y * np.float32(2.0 ** k)                                 # exact unless it overflows to infinity
+    return _round_to_int(z, np.int32)
+
+
+def bf16_scaled_round(bits, k, dtype):
+    """(p.to(float32) * 2**k).round().to(dtype) for bfloat16 bit patterns (inference/convert2.py:250-262, 290-295)"""
+    x = (np.ascontiguousarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        z = x * np.float32(2.0 ** k)
+    return _round_to_int(z, dtype)
+
+
 def float32_to_int64_2d(bits, rescale):
     bits = _c(bits, np.uint32)
     out = np.empty(bits.shape, np.int64)

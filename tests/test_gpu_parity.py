@@ -837,3 +837,32 @@ def test_converters(K, oracle):
     want = oracle.float32_to_int64_2d(big32.cpu().numpy().view(np.uint32)[1:].reshape(1, n), 12)
     assert np.array_equal(host(out64)[1:], want.ravel())
     K._check("converters")
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (300, 520), (1, 129), (129, 1), (7, 2048), (2048, 7168)])
+def test_fp8_checkpoint_quantisation(K, oracle, shape):
+    """block-scaled fp8 weights -> int32 fixed point in one pass (convert2.py:144-147): every fp8 code incl. NaN,
+    scales from 2^-20 to 4, ragged block edges, values that saturate"""
+    rows, cols = shape
+    rng = np.random.default_rng(rows + cols)
+    w = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    w[0, : min(cols, 256)] = np.arange(min(cols, 256), dtype=np.uint8)
+    sc = np.exp2(rng.uniform(-20, 2, ((rows + 127) // 128, (cols + 127) // 128))).astype(np.float32)
+    wd, sd = dev(w), dev(sc)
+    for k in ((0, 21, 30) if rows * cols < (1 << 22) else (30,)):
+        assert np.array_equal(host(K.quantize_fp8_weight(wd, sd, k)), oracle.fp8_block_scaled_to_int32(w, sc, k))
+    assert np.array_equal(host(K.quantize_fp8_weight(wd.view(torch.float8_e4m3fn), sd, 25)), oracle.fp8_block_scaled_to_int32(w, sc, 25))
+
+
+def test_bf16_checkpoint_quantisation(K, oracle):
+    """(p.float() * 2^k).round() to int32 / int64 for every bfloat16 pattern (convert2.py:250-262, 290-295)"""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    pd = dev(bits.view(np.int16)).view(torch.bfloat16)
+    for k in (0, 1, 15, 21, 31, 43, 127):
+        assert np.array_equal(host(K.quantize_bf16(pd, k, torch.int32)), oracle.bf16_scaled_round(bits, k, np.int32))
+        assert np.array_equal(host(K.quantize_bf16(pd, k, torch.int64)), oracle.bf16_scaled_round(bits, k, np.int64))
+    out = torch.empty((4,), dtype=torch.int32, device="cuda")
+    K.lib.bf16_scaled_round_to_int32(pd.data_ptr(), out.data_ptr(), 4, 128)
+    assert K.lib.zk_last_error() == 1
+    K.lib.zk_clear_error()
+

@@ -354,6 +354,46 @@ def _route_numpy(scores, bias, n_groups, topk_groups, topk):
     return w * 5 // 2, idx, raw
 
 
+def test_checkpoint_quantisation_equals_the_tensor_ops_it_restates(oracle):
+    """fp8_block_scaled_to_int32 / bf16_scaled_round against torch's own CPU tensor ops, written as convert2.py writes
+    them (inference/convert2.py:144-147, 250-262) with the Triton kernel's three operations (kernel.py:90-93: load
+    as float32, multiply by the block scale, store as bfloat16) as tensor ops: every fp8 code, scales from tiny to
+    large, ragged block edges, ties of both roundings."""
+    import torch
+    rng = np.random.default_rng(8)
+    tab = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    mine = oracle._e4m3fn_table()
+    assert np.array_equal(np.isnan(tab), np.isnan(mine)) and np.array_equal(tab[~np.isnan(tab)], mine[~np.isnan(mine)])
+    for rows, cols in ((256, 256), (300, 520), (1, 129), (129, 1)):
+        w = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+        w[0, : min(cols, 256)] = np.arange(min(cols, 256), dtype=np.uint8)
+        sc = np.exp2(rng.uniform(-20, 2, ((rows + 127) // 128, (cols + 127) // 128))).astype(np.float32)
+        for k in (0, 7, 21, 30):
+            x = torch.from_numpy(w).view(torch.float8_e4m3fn).to(torch.float32)
+            s = torch.from_numpy(sc).repeat_interleave(128, 0).repeat_interleave(128, 1)[:rows, :cols]
+            z = ((x * s).to(torch.bfloat16).to(torch.float32) * (2 ** k)).round()
+            inside = (~torch.isnan(z)) & (z.abs() < 2.0 ** 31)
+            want = z[inside].to(torch.int32).numpy()
+            got = oracle.fp8_block_scaled_to_int32(w, sc, k)
+            assert np.array_equal(got[inside.numpy()], want)
+            assert np.all(got[torch.isnan(z).numpy()] == 0)
+            assert np.all(got[(z >= 2.0 ** 31).numpy()] == 2 ** 31 - 1) and np.all(got[(z <= -(2.0 ** 31)).numpy()] == -(2 ** 31))
+    # every bfloat16 pattern, both widths; k = 0 and 1 put values exactly on .5 (round half to even)
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    pt = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    for k in (0, 1, 15, 31, 43):
+        z = (pt.to(torch.float32) * (2 ** k)).round()
+        for dt, tdt, lim in ((np.int32, torch.int32, 2.0 ** 31), (np.int64, torch.int64, 2.0 ** 63)):
+            inside = (~torch.isnan(z)) & (z.abs() < lim)
+            got = oracle.bf16_scaled_round(bits, k, dt)
+            assert np.array_equal(got[inside.numpy()], z[inside].to(tdt).numpy())
+            assert np.all(got[torch.isnan(z).numpy()] == 0)
+    assert oracle.bf16_scaled_round(np.array([0x3F00, 0x3FC0, 0x4020, 0xBF00, 0xBFC0], np.uint16), 0, np.int32).tolist() == [0, 2, 2, 0, -2]
+    # ties of the bfloat16 store: 1 + 2^-8 is halfway between 1 and 1 + 2^-7 -> even (1); 1 + 3*2^-8 -> 1 + 2^-6
+    y = oracle._round_to_bf16(np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, -(1 + 2.0 ** -8)], np.float32))
+    assert y.tolist() == [1.0, 1 + 2.0 ** -6, -1.0]
+
+
 @pytest.mark.parametrize("E,G,KG,K", [(256, 8, 4, 8), (16, 4, 2, 4), (64, 1, 1, 6), (96, 3, 3, 5), (512, 8, 3, 8)])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gate_route_matches_the_tensor_op_restatement(oracle, E, G, KG, K, with_bias):

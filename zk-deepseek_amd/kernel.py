@@ -54,6 +54,9 @@ for _n in ("silu_q25", "sigmoid_q25", "silu_q23", "sigmoid_q23"):
 for _n in ("bf16_to_int32_2d", "float32_to_int64_2d"):
     getattr(lib, _n).argtypes = [_vp, _vp, _ci, _ci, _ci]
 lib.wkv_b_bf16_to_int32.argtypes = [_vp, _vp, _ci, _ci]
+lib.fp8_block_scaled_to_int32.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci]
+lib.bf16_scaled_round_to_int32.argtypes = [_vp, _vp, ctypes.c_long, _ci]
+lib.bf16_scaled_round_to_int64.argtypes = [_vp, _vp, ctypes.c_long, _ci]
 # additions without a reference counterpart
 lib.rms_stat_int64.argtypes = [_vp, _vp, _ci, _ci, _ll, _ll]
 lib.rms_norm_fused_32.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
@@ -259,6 +262,34 @@ def RMS_Norm_residual_int64(X: torch.Tensor, Y: torch.Tensor, k: int, W: torch.T
     _check("RMS_Norm_residual_int64")
     rms[:M] = rms_gpu[:M].cpu()
     return (Xout, C, rms)
+
+
+def quantize_fp8_weight(weight: torch.Tensor, scale: torch.Tensor, k: int) -> torch.Tensor:
+    """int32 fixed-point weights from a block-scaled fp8 checkpoint tensor, in one pass on the device:
+    (weight_dequant(weight, scale).to(float32) * 2**k).round().to(int32) of inference/convert2.py:144-147
+    (weight_dequant: inference/kernel.py:96-117, 128x128 blocks, bfloat16 result).
+    weight [rows, cols] float8_e4m3fn (or its bytes as uint8), scale [ceil(rows/128), ceil(cols/128)] float32."""
+    assert weight.is_cuda and scale.is_cuda and weight.is_contiguous() and scale.is_contiguous()
+    assert weight.dim() == 2 and scale.dim() == 2
+    assert weight.dtype in (torch.float8_e4m3fn, torch.uint8) and scale.dtype == torch.float32
+    rows, cols = weight.shape
+    assert scale.shape == ((rows + 127) // 128, (cols + 127) // 128)
+    out = torch.empty((rows, cols), dtype=torch.int32, device=weight.device)
+    lib.fp8_block_scaled_to_int32(weight.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, cols, k)
+    _check("quantize_fp8_weight")
+    return out
+
+
+def quantize_bf16(param: torch.Tensor, k: int, dtype=torch.int32) -> torch.Tensor:
+    """(param.to(float32) * 2**k).round().to(dtype) for a bfloat16 tensor (inference/convert2.py:250-262, 290-295,
+    353-359), dtype int32 or int64."""
+    assert param.is_cuda and param.is_contiguous() and param.dtype == torch.bfloat16
+    assert dtype in (torch.int32, torch.int64)
+    out = torch.empty(param.shape, dtype=dtype, device=param.device)
+    fn = lib.bf16_scaled_round_to_int32 if dtype == torch.int32 else lib.bf16_scaled_round_to_int64
+    fn(param.data_ptr(), out.data_ptr(), param.numel(), k)
+    _check("quantize_bf16")
+    return out
 
 
 atexit.register(lambda: lib.zk_dump_flush())
