@@ -7,6 +7,12 @@ module) never imports this file.
 All functions take and return C-contiguous numpy arrays and mirror the Python
 operator API of the reference's inference/kernel.py:341-688 (same argument
 order and meaning), except that nothing lives on a GPU.
+
+Functions below that are compositions in numpy (the fusions, the MoE path, the checkpoint quantisation) restate
+tensor ops of inference/model.py and inference/convert2.py, cited where they are defined.  Parity unpinned (the
+reference leaves them to its device, and nothing it ships can confirm the choice made here): float values outside
+the integer range and NaN in the checkpoint quantisation (fixed as saturation and 0); see zk_oracle.c for the
+integer kernels' list.
 """
 import ctypes
 import os
