@@ -337,6 +337,16 @@ def main():
         finally:
             shutil.rmtree(tmpd, ignore_errors=True)
 
+        # config 2's GEMMs (one expert FFN at M = 128): w1/w3 [2048,7168] and w2 [7168,2048], shift 16
+        g2m = torch.Generator(device="cpu").manual_seed(2000)
+        X2 = randint(g2m, -(1 << 20), 1 << 20, (1, 128, 7168)).cuda()
+        W21 = randint(g2m, -(1 << 16), 1 << 16, (2048, 7168)).cuda()
+        H2 = randint(g2m, -(1 << 20), 1 << 20, (1, 128, 2048)).cuda()
+        W22 = randint(g2m, -(1 << 16), 1 << 16, (7168, 2048)).cuda()
+        extra["gemm_config2_w1_128x7168x2048"] = gemm_leg(K, X2, W21, 16, 50, 5)
+        extra["gemm_config2_w2_128x2048x7168"] = gemm_leg(K, H2, W22, 16, 50, 5)
+        del X2, W21, H2, W22
+
         # the four MLA einsums at config 3's shape (S = T = 1024, 128 heads, absorb mode: model.py:884-936), Q30
         # activations against Q24 cache entries / int32 Q25 weights
         ge = torch.Generator(device="cuda").manual_seed(900)
@@ -362,6 +372,14 @@ def main():
         pp = torch.randint(0, 1 << 19, (1, Se, He, Se), generator=ge, dtype=torch.int64, device="cuda")
         einsum_leg("einsum_bsht_btc_bshc_1x1024x128xT1024_to_512", lambda: K.einsum_bsht_btc_bshc(pp, kvc, 23), Se * He * Se * Ce)
         del pp, kvc
+        # config 3 as BASELINE states it: Q [1,1024,128,192] against K [1,1024,192] in one call, P.V with 128 columns
+        q3, k3 = rnd(16, 1, Se, He, 192), rnd(16, 1, Se, 192)
+        einsum_leg("einsum_bshc_btc_bsht_config3_1x1024x128x192_T1024", lambda: K.einsum_bshc_btc_bsht(q3, k3, 21), Se * He * Se * 192)
+        del q3, k3
+        p3 = torch.randint(0, 1 << 19, (1, Se, He, Se), generator=ge, dtype=torch.int64, device="cuda")
+        v3 = rnd(16, 1, Se, 128)
+        einsum_leg("einsum_bsht_btc_bshc_config3_1x1024x128xT1024_to_128", lambda: K.einsum_bsht_btc_bshc(p3, v3, 23), Se * He * Se * 128)
+        del p3, v3
         oo, wb2 = rnd(30, 1, Se, He, Ce), rnd(25, He, De, Ce).to(torch.int32)
         einsum_leg("einsum_bshc_hdc_bshd_1x1024x128x512_to_128", lambda: K.einsum_bshc_hdc_bshd(oo, wb2, 21), Se * He * De * Ce)
         del oo, wb2

@@ -319,7 +319,13 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
 
 // Folds the per-workgroup ranges of the plane pre-pass (`mm`, A only) and of the GEMM kernel (`wg`, A and B) into
 // range[0..3] and leaves the verdict in range[4]: 0 when `na` and `nb` digits covered them, 1 otherwise.
-// `host_copy`, when set, is pinned host memory that receives the same five words.  One workgroup of any size.
+// `host_copy`, when set, is pinned host memory that receives the same five words.
+// `parts` workgroups (of any size) share the slots; each leaves its partial result in `scratch` and takes a ticket, and
+// the one that arrives last folds the partials (a launch with tens of thousands of tiles would otherwise spend longer
+// in a one-workgroup fold than some GEMMs take).  range[5] is the ticket counter; it is zero between launches.
+constexpr int kFoldParts = 64;        // at most this many workgroups fold
+constexpr long kFoldSlotsPerPart = 1024;
+
 struct FoldArgs {
     const unsigned long long *mm;
     long mm_count;
@@ -328,60 +334,70 @@ struct FoldArgs {
     unsigned long long *range;
     int na, nb;
     unsigned long long *host_copy;
+    int parts;
+    unsigned long long *scratch;      // 4 * kFoldParts words
 };
 
-__device__ __forceinline__ void range_fold_body(const FoldArgs &f)
+__host__ __device__ inline unsigned long long fold_pick(int q, unsigned long long a, unsigned long long b)
+{
+    return (q & 1) ? (a > b ? a : b) : (a < b ? a : b);       // words 1 and 3 are maxima, 0 and 2 minima
+}
+
+__device__ __forceinline__ void range_fold_body(const FoldArgs &f, int part)
 {
     __shared__ unsigned long long red[16][4];
     const int nthreads = blockDim.x;
+    const long first = (long)part * nthreads + threadIdx.x, stride = (long)f.parts * nthreads;
     unsigned long long v[4] = { ~0ull, 0ull, ~0ull, 0ull };
-    for (long i = threadIdx.x; i < f.mm_count; i += nthreads) {
-        const unsigned long long a = f.mm[2 * i], b = f.mm[2 * i + 1];
-        v[0] = a < v[0] ? a : v[0];
-        v[1] = b > v[1] ? b : v[1];
+    for (long i = first; i < f.mm_count; i += stride) {
+        v[0] = fold_pick(0, f.mm[2 * i], v[0]);
+        v[1] = fold_pick(1, f.mm[2 * i + 1], v[1]);
     }
-    for (long i = threadIdx.x; i < f.wg_count; i += nthreads) {
+    for (long i = first; i < f.wg_count; i += stride) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const unsigned long long a = f.wg[4 * i + q];
-            v[q] = (q & 1) ? (a > v[q] ? a : v[q]) : (a < v[q] ? a : v[q]);
-        }
+        for (int q = 0; q < 4; q++) v[q] = fold_pick(q, f.wg[4 * i + q], v[q]);
     }
 #pragma unroll
     for (int q = 0; q < 4; q++) {
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const unsigned long long o = (unsigned long long)__shfl_xor((long long)v[q], off, kWave);
-            v[q] = (q & 1) ? (o > v[q] ? o : v[q]) : (o < v[q] ? o : v[q]);
-        }
+        for (int off = 32; off > 0; off >>= 1)
+            v[q] = fold_pick(q, (unsigned long long)__shfl_xor((long long)v[q], off, kWave), v[q]);
     }
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
         for (int q = 0; q < 4; q++) red[threadIdx.x >> 6][q] = v[q];
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < nthreads / 64; w++)
+    if (threadIdx.x != 0) return;
+    for (int w = 1; w < nthreads / 64; w++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const unsigned long long o = red[w][q];
-                v[q] = (q & 1) ? (o > v[q] ? o : v[q]) : (o < v[q] ? o : v[q]);
-            }
+        for (int q = 0; q < 4; q++) v[q] = fold_pick(q, red[w][q], v[q]);
+    if (f.parts > 1) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) f.range[q] = v[q];
-        const int need_a = limbs_needed((int64_t)(v[0] ^ kSignFlip), (int64_t)(v[1] ^ kSignFlip));
-        const int need_b = limbs_needed((int64_t)(v[2] ^ kSignFlip), (int64_t)(v[3] ^ kSignFlip));
-        const unsigned long long verdict = (need_a <= f.na && need_b <= f.nb) ? 0ull : 1ull;
-        f.range[4] = verdict;
-        if (f.host_copy) {
+        for (int q = 0; q < 4; q++) __hip_atomic_store(&f.scratch[4 * part + q], v[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // release the partial, then count in; whoever sees everyone else counted in acquires their partials
+        const unsigned long long ticket = __hip_atomic_fetch_add(&f.range[5], 1ull, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (ticket != (unsigned long long)(f.parts - 1)) return;
+        for (int w = 0; w < f.parts; w++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) f.host_copy[q] = v[q];
-            f.host_copy[4] = verdict;
-        }
+            for (int q = 0; q < 4; q++)
+                v[q] = fold_pick(q, __hip_atomic_load(&f.scratch[4 * w + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), v[q]);
+        __hip_atomic_store(&f.range[5], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) f.range[q] = v[q];
+    const int need_a = limbs_needed((int64_t)(v[0] ^ kSignFlip), (int64_t)(v[1] ^ kSignFlip));
+    const int need_b = limbs_needed((int64_t)(v[2] ^ kSignFlip), (int64_t)(v[3] ^ kSignFlip));
+    const unsigned long long verdict = (need_a <= f.na && need_b <= f.nb) ? 0ull : 1ull;
+    f.range[4] = verdict;
+    if (f.host_copy) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) f.host_copy[q] = v[q];
+        f.host_copy[4] = verdict;
     }
 }
 
-__global__ __launch_bounds__(256) void range_fold_kernel(FoldArgs f) { range_fold_body(f); }
+__global__ __launch_bounds__(256) void range_fold_kernel(FoldArgs f) { range_fold_body(f, (int)blockIdx.x); }
 
 // Number of digit pairs (i', j') with i' + j' < d that come before (i, j) in row order (i' < i, or i' == i and j' < j).
 __host__ __device__ constexpr int kept_pairs_before(int na, int nb, int d, int i, int j)
@@ -749,58 +765,77 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
     // epilogue: diagonals -> 128-bit sum -> shift.  Accumulator register r of lane l holds
     // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile.
-    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+    // Diagonals are added in groups of four: a group's sum of v[4g+j] * 2^(8j) stays below 2^57, so it is plain 64-bit
+    // arithmetic; the groups (weights 2^0, 2^32, 2^64, 2^96) then meet in one 128-bit sum.
+    auto combine = [&](int a, int b, int r, u128 sum) {
 #pragma unroll
-    for (int a = 0; a < WM; a++) {
+        for (int gq = 0; gq < (D + 3) / 4; gq++) {
+            uint64_t s = (uint64_t)(int64_t)acc[a][b][4 * gq][r];
 #pragma unroll
-        for (int b = 0; b < WN; b++) {
-            const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
+            for (int j = 1; j < 4; j++)
+                if (4 * gq + j < D) s += (uint64_t)(int64_t)acc[a][b][4 * gq + j][r] << (8 * j);
+            sum += (u128)(i128)(int64_t)s << (32 * gq);
+        }
+        return sum;
+    };
+    if (nsplit > 1) {
+        // raw partial sums (without the rounding term), finished by gemm_split_finish_kernel: 64 lanes' low words, then
+        // (unless 64 bits hold the sums) their high words, per (slice, wave, tile, register)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                // rows of this register that all lie past M (uniform over the wave): nothing to keep
-                if (nsplit > 1 && m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= m_lim) continue;
-                // whole tiles start from the rounding term; split workgroups leave it to the finishing kernel
-                uint64_t lo = nsplit > 1 ? 0 : (uint64_t)p.init, hi = nsplit > 1 ? 0 : (uint64_t)(p.init >> 63);
+        for (int a = 0; a < WM; a++)
 #pragma unroll
-                for (int d = 0; d < D; d++) {
-                    const int64_t v = (int64_t)acc[a][b][d][r];
-                    uint64_t clo, chi;
-                    if (d == 0) { clo = (uint64_t)v; chi = (uint64_t)(v >> 63); }
-                    else if (d < 8) { clo = (uint64_t)v << (8 * d); chi = (uint64_t)(v >> (64 - 8 * d)); }
-                    else if (d == 8) { clo = 0; chi = (uint64_t)v; }
-                    else { clo = 0; chi = (uint64_t)v << (8 * (d - 8)); }
-                    const uint64_t s = lo + clo;
-                    hi += chi + (s < lo ? 1 : 0);
-                    lo = s;
-                }
-                if (nsplit > 1) {
-                    // raw partial sum (without init), finished by gemm_split_finish_kernel: 64 lanes' low words, then
-                    // (unless 64 bits hold the sums) their high words, per (slice, wave, tile, register)
+            for (int b = 0; b < WN; b++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    // rows of this register that all lie past M (uniform over the wave): nothing to keep
+                    if (m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= m_lim) continue;
+                    const u128 sum = combine(a, b, r, 0);
                     const long q = (((long)tail_tile * p.split + sidx) * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r;
-                    if (p.part64) p.partials[q * 64 + lane] = lo;
-                    else { p.partials[q * 128 + lane] = lo; p.partials[q * 128 + 64 + lane] = hi; }
-                } else if (m < m_lim && n < p.N) {
-                    const long o = (long)g * p.sC + (long)m * p.ldc + n;
-                    uint64_t q;
-                    if (p.shift == 0) q = lo;
-                    else q = (lo >> p.shift) | (hi << (64 - p.shift));
-                    p.C[o] = (int64_t)q;
-                    if (p.R) p.R[o] = (int64_t)(lo & rmask);
+                    if (p.part64) p.partials[q * 64 + lane] = (uint64_t)sum;
+                    else { p.partials[q * 128 + lane] = (uint64_t)sum; p.partials[q * 128 + 64 + lane] = (uint64_t)(sum >> 64); }
+                }
+        return;
+    }
+    // Whole tiles: the loops carry no uniform branches (tiles that reach past M or N, and calls that want the remainder,
+    // have their own copy), and a row's address is the tile's plus a scalar multiple of the row stride.
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+    const u128 sum0 = (u128)(i128)p.init;
+    const int sh = p.shift;
+    auto store_tile = [&](auto edge_tag, auto rem_tag) {
+        constexpr bool EDGE = decltype(edge_tag)::value, REM = decltype(rem_tag)::value;
+#pragma unroll
+        for (int a = 0; a < WM; a++)
+#pragma unroll
+            for (int b = 0; b < WN; b++) {
+                const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
+                const int mrow = m0 + (wm * WM + a) * 32 + 4 * (lane >> 5);
+                const long o0 = (long)g * p.sC + (long)mrow * p.ldc + n;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int dr = 8 * (r >> 2) + (r & 3);
+                    const u128 sum = combine(a, b, r, sum0);
+                    const uint64_t lo = (uint64_t)sum, hi = (uint64_t)(sum >> 64);
+                    if (EDGE && !(mrow + dr < m_lim && n < p.N)) continue;
+                    const long o = o0 + (long)dr * p.ldc;
+                    // bits [sh, sh + 64): the upper word comes in through two shifts so that sh == 0 needs no case of its own
+                    p.C[o] = (int64_t)((lo >> sh) | ((hi << 1) << (63 - sh)));
+                    if (REM) p.R[o] = (int64_t)(lo & rmask);
                 }
             }
-        }
-    }
+    };
+    const bool edge = m0 + BM > m_lim || n0 + BN > p.N;
+    if (p.R) { if (edge) store_tile(std::true_type(), std::true_type()); else store_tile(std::false_type(), std::true_type()); }
+    else { if (edge) store_tile(std::true_type(), std::false_type()); else store_tile(std::false_type(), std::false_type()); }
 }
 
 // Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
 // Thread layout and element order are those of the GEMM kernel's epilogue.
-// The workgroup behind the last one folds the ranges (the GEMM kernel has left them by then), which saves a launch.
+// The last `fold.parts` workgroups fold the ranges (the GEMM kernel has left them by then), which saves a launch.
 template <int WVM, int WVN, int WM, int WN>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaParams p, FoldArgs fold)
 {
-    if (blockIdx.x == gridDim.x - 1) {
-        range_fold_body(fold);
+    if (blockIdx.x >= gridDim.x - fold.parts) {
+        range_fold_body(fold, (int)(blockIdx.x - (gridDim.x - fold.parts)));
         return;
     }
     constexpr int T = 64 * WVM * WVN, BM = 32 * WM * WVM, BN = 32 * WN * WVN;
@@ -1045,8 +1080,11 @@ long gemm_mfma_guard_hits()
 static bool init_cache()
 {
     if (g_cache.dev) return true;
-    if (hipMalloc(&g_cache.dev, 8 * sizeof(unsigned long long)) != hipSuccess) {
-        set_error(kLaunchFailure, "gemm: cannot allocate the 64-byte range buffer");
+    // [minA, maxA, minB, maxB, verdict, fold ticket, -, -] and the partial results of the folding workgroups
+    const size_t dev_bytes = (8 + 4 * kFoldParts) * sizeof(unsigned long long);
+    if (hipMalloc(&g_cache.dev, dev_bytes) != hipSuccess || hipMemset(g_cache.dev, 0, dev_bytes) != hipSuccess) {
+        g_cache.dev = nullptr;
+        set_error(kLaunchFailure, "gemm: cannot allocate the range buffer");
         return false;
     }
     int dev = 0, n = 0;
@@ -1063,6 +1101,14 @@ static bool init_cache()
         g_cache.pinned = nullptr;
     }
     return true;
+}
+
+static FoldArgs make_fold(const unsigned long long *mm, long mm_count, const unsigned long long *wg, long wg_count,
+                          unsigned long long *range, int na, int nb, unsigned long long *host_copy)
+{
+    long parts = (mm_count + wg_count + kFoldSlotsPerPart - 1) / kFoldSlotsPerPart;
+    parts = parts < 1 ? 1 : (parts > kFoldParts ? kFoldParts : parts);
+    return FoldArgs{ mm, mm_count, wg, wg_count, range, na, nb, host_copy, (int)parts, g_cache.dev + 8 };
 }
 
 bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
@@ -1224,12 +1270,12 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                 return false;
             }
         }
-        const FoldArgs fold = { g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb, slot ? slot->host : nullptr };
+        const FoldArgs fold = make_fold(g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb, slot ? slot->host : nullptr);
         if (p.split > 1) {
-            inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq + 1)), dim3((unsigned)inst->threads), 0, 0>>>(p, fold);
+            inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq + fold.parts)), dim3((unsigned)inst->threads), 0, 0>>>(p, fold);
             if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
         } else {
-            range_fold_kernel<<<1, 256, 0, 0>>>(fold);
+            range_fold_kernel<<<dim3((unsigned)fold.parts), 256, 0, 0>>>(fold);
         }
         *limbs_a = inst->na;
         *limbs_b = inst->nb;
@@ -1317,7 +1363,8 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
                 return -1;
             }
         }
-        range_fold_kernel<<<1, 256, 0, 0>>>(FoldArgs{ nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr });
+        const FoldArgs fold = make_fold(nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr);
+        range_fold_kernel<<<dim3((unsigned)fold.parts), 256, 0, 0>>>(fold);
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "grouped gemm: range readback failed"); return -1; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
