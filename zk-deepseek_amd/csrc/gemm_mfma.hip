@@ -63,6 +63,7 @@ struct MfmaParams {
     // split-K tail: workgroup ids below main_tiles are whole tiles; the rest are `split` workgroups per tile that
     // each cover a slice of K and leave raw 128-bit partial sums in `partials`
     int main_tiles, split;
+    int n_fastest;                            // tile order inside a batch: 0 = tile rows move fastest (the workgroups that run together share a B tile), 1 = tile columns (they share an A tile)
     unsigned long long *partials;
     int part64;                     // the partial sums fit 64 bits: only the low words are kept
     // grouped mode (GRP kernels): rows of A and C form one segment per group, each group has its own B.
@@ -474,8 +475,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         tail_tile = lin - p.main_tiles;            // index among the split tiles (when nsplit > 1)
         g = lin / per_batch;
         const int rem = lin - g * per_batch;
-        tn = rem / p.tiles_m;
-        tm = rem - tn * p.tiles_m;
+        if (p.n_fastest) { tm = rem / p.tiles_n; tn = rem - tm * p.tiles_n; }
+        else { tn = rem / p.tiles_m; tm = rem - tn * p.tiles_m; }
         m0 = tm * BM;
     }
     const int n0 = tn * BN;
@@ -845,7 +846,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
     const int tail_tile = blockIdx.x / p.finish_rq, rq = blockIdx.x % p.finish_rq, lin = p.main_tiles + tail_tile;
     const int r_per = 16 / p.finish_rq;
     const int g = lin / per_batch, rem = lin - g * per_batch;
-    const int tn = rem / p.tiles_m, tm = rem - tn * p.tiles_m;
+    const int tn = p.n_fastest ? rem % p.tiles_n : rem / p.tiles_m, tm = p.n_fastest ? rem / p.tiles_n : rem - tn * p.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
     const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
 #pragma unroll
@@ -1175,6 +1176,10 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         const int BM = inst->bm, BN = inst->bn;
         p.tiles_m = (d.M + BM - 1) / BM;
         p.tiles_n = (d.N + BN - 1) / BN;
+        // A B operand that stays in L2 whatever the order (the MLA einsums: a KV cache or one head's weights against
+        // a hundred thousand rows) lets the tile columns move fastest, so that each A tile is streamed once
+        const size_t b_bytes = (size_t)d.N * d.K * (d.b32 ? 4 : 8);
+        p.n_fastest = (b_bytes <= ((size_t)8 << 20) && p.tiles_n > 1 && p.tiles_m > 1) ? 1 : 0;
         const long per_batch = (long)p.tiles_m * p.tiles_n;
         if (per_batch > 0x7FFFFFFFL) return false;
         const long total = per_batch * d.G;
