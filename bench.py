@@ -208,6 +208,11 @@ def main():
             hbm("softmax_q19_1x%dx128x1024" % S,
                 lambda: K.lib.softmax_q19(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q19.data_ptr(), 1, S, 128, 1024),
                 R.numel(), steps=10)
+            if S == 1024:       # the Q21 variant (no live caller in the reference's model) on the same rows
+                K.softmax_init_q21()
+                hbm("softmax_q21_1x1024x128x1024",
+                    lambda: K.lib.softmax_q21(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q21.data_ptr(), 1, S, 128, 1024),
+                    R.numel(), steps=10)
             del R, Cs
         for S in (512, 8192):
             g2 = torch.Generator(device="cpu").manual_seed(2300 + S)
@@ -217,6 +222,12 @@ def main():
                 hbm("%s_1x%dx18432" % (nm, S),
                     lambda fn=fn: fn(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q23.data_ptr(), 1, S, 18432),
                     R.numel(), steps=20)
+            if S == 8192:       # the Q25 variants (bound at import only in the reference)
+                K.silu_init_q25()
+                for nm, fn in (("silu_q25", K.lib.silu_q25), ("sigmoid_q25", K.lib.sigmoid_q25)):
+                    hbm("%s_1x%dx18432" % (nm, S),
+                        lambda fn=fn: fn(R.data_ptr(), Cs.data_ptr(), K.EXP2_FRAC_LUT_Q25.data_ptr(), 1, S, 18432),
+                        R.numel(), steps=20)
             del R, Cs
         g6 = torch.Generator(device="cpu").manual_seed(600)
         for Mr in (500, 16384):
