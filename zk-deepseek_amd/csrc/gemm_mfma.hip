@@ -63,6 +63,7 @@ struct MfmaParams {
     // split-K tail: workgroup ids below main_tiles are whole tiles; the rest are `split` workgroups per tile that
     // each cover a slice of K and leave raw 128-bit partial sums in `partials`
     int main_tiles, split;
+    int tail_xcd;                             // split tiles: deal (tile column, K slice) pairs over the 8 XCDs (see the kernel)
     int n_fastest;                            // tile order inside a batch: 0 = tile rows move fastest (the workgroups that run together share a B tile), 1 = tile columns (they share an A tile)
     unsigned long long *partials;
     int part64;                     // the partial sums fit 64 bits: only the low words are kept
@@ -468,8 +469,17 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             if ((p.main_tiles & 7) == 0) lin = (lin & 7) * (p.main_tiles >> 3) + (lin >> 3);
         } else {
             const int t = lin - p.main_tiles;
-            lin = p.main_tiles + t / p.split;
-            sidx = t % p.split;
+            if (p.tail_xcd) {
+                // Workgroup ids go round the 8 XCDs.  Each XCD takes whole (tile column, K slice) pairs and runs the
+                // tiles_m workgroups of a pair one after the other, so that they find the pair's B data in their L2.
+                const int x = t & 7, q = t >> 3;
+                const int pair = (q / p.tiles_m) * 8 + x;
+                lin = p.main_tiles + (pair / p.split) * p.tiles_m + q % p.tiles_m;
+                sidx = pair % p.split;
+            } else {
+                lin = p.main_tiles + t / p.split;
+                sidx = t % p.split;
+            }
             nsplit = p.split;
         }
         tail_tile = lin - p.main_tiles;            // index among the split tiles (when nsplit > 1)
@@ -1201,6 +1211,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         int tail = (int)(total % g_cache.cus), split = 1;
         p.main_tiles = (int)total;
         p.split = 1;
+        p.tail_xcd = 0;
         p.partials = nullptr;
         p.part64 = 0;
         p.finish_rq = 4;
@@ -1234,6 +1245,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             if (grow(g_cache.partials, g_cache.partials_bytes, need, "partial-sum buffer")) {
                 p.main_tiles = (int)(total - tail);
                 p.split = split;
+                p.tail_xcd = (!p.n_fastest && d.G == 1 && tail % p.tiles_m == 0 && p.main_tiles % 8 == 0 &&
+                              ((long)tail * split) % (8L * p.tiles_m) == 0) ? 1 : 0;
                 p.partials = g_cache.partials;
                 p.part64 = part64 ? 1 : 0;
             } else if (zk_last_error() != kOk) return false;
