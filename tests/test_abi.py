@@ -108,3 +108,20 @@ def test_dump_writer_host_path(lib, tmp_path):
     assert b"no_such_dir" in lib.zk_last_error_string()
     lib.zk_clear_error()
     assert lib.zk_dump_flush() == 0
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """the boundary is a C ABI: the header compiles as C99 with gcc (no C++, no HIP types), and a C program that takes
+    the address of every declared function links against the library and runs without a GPU"""
+    import subprocess
+    names = declared_functions()
+    src = tmp_path / "abi.c"
+    body = "".join("    keep[%d] = (fn_t)&%s;\n" % (i, n) for i, n in enumerate(names))
+    src.write_text('#include "int64gemm.h"\n#include <stdio.h>\ntypedef void (*fn_t)(void);\nint main(void) {\n'
+                   '    fn_t keep[%d];\n%s    printf("%%d %%d\\n", keep[0] != 0, zk_last_error());\n    return 0;\n}\n' % (len(names), body))
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(LIB)
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.dirname(HEADER),
+                           str(src), "-o", str(exe), "-L", libdir, "-lint64gemm", "-Wl,-rpath," + libdir,
+                           "-Wl,-rpath-link,/opt/rocm/lib"])
+    assert subprocess.check_output([str(exe)]).decode().split() == ["1", "0"]
