@@ -110,7 +110,7 @@ def test_dump_writer_host_path(lib, tmp_path):
     assert lib.zk_dump_flush() == 0
 
 
-def test_header_is_plain_c_and_links(tmp_path):
+def test_header_is_plain_c_and_links(lib, tmp_path):
     """the boundary is a C ABI: the header compiles as C99 with gcc (no C++, no HIP types), and a C program that takes
     the address of every declared function links against the library and runs without a GPU"""
     import subprocess
