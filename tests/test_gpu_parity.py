@@ -206,6 +206,58 @@ def test_gemm_config4_full_size_sampled(K, oracle, path, full_range):
     assert torch.equal(C1, torch.roll(C0, 1, dims=1))
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_gemm_seeded_random_problems(K, oracle, seed):
+    """a sweep no hand-picked list would make: random batch, shape, operand widths, weight type and shift per case, on
+    the MFMA path (whole tiles, edge tiles, 32-row tiles, K split, digit planes or not, few or many diagonals kept)"""
+    rng = np.random.default_rng(9000 + seed)
+    for _ in range(6):
+        Bd = int(rng.choice([1, 1, 2, 3]))
+        M = int(rng.choice([1, 5, 16, 31, 33, 64, 100, 129, 200, 300]))
+        Kd = int(rng.choice([1, 7, 32, 33, 96, 250, 512, 1000, 2048]))
+        N = int(rng.choice([1, 9, 64, 127, 130, 256, 520, 1100]))
+        while Bd * M * Kd * N > 60_000_000:         # keep the scalar oracle to a fraction of a second per case
+            Kd = max(1, Kd // 2)
+        w32 = bool(rng.integers(0, 2))
+        bits_a = int(rng.choice([3, 12, 20, 31, 37, 47, 56, 63]))
+        bits_w = int(rng.choice([3, 12, 16, 24, 31])) if w32 else int(rng.choice([3, 16, 24, 33, 47, 63]))
+        c = int(rng.choice([0, 1, 8, 16, 23, 29, 31, 32, 33, 40, 63]))
+        A = rand_i64(rng, (Bd, M, Kd), bits_a)
+        W = rand_i32(rng, (N, Kd), bits_w) if w32 else rand_i64(rng, (N, Kd), bits_w)
+        try:
+            _gemm_case(K, oracle, 2, A, W, 1, 1, c)
+        except AssertionError as e:
+            raise AssertionError("%s for B=%d M=%d K=%d N=%d w32=%s bits=(%d,%d) c=%d" % (e, Bd, M, Kd, N, w32, bits_a, bits_w, c))
+    K.lib.zk_gemm_set_path(0)
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_einsums_seeded_random_problems(K, oracle, seed):
+    """the four einsums on random shapes and operand widths (strided A rows, k-major and int32 B, per-head batches)"""
+    rng = np.random.default_rng(9500 + seed)
+    for _ in range(3):
+        B = int(rng.choice([1, 2]))
+        S = int(rng.choice([1, 7, 40, 130]))
+        H = int(rng.choice([1, 3, 16]))
+        D = int(rng.choice([8, 24, 64, 128]))
+        Cc = int(rng.choice([16, 40, 64, 192, 512]))
+        T = int(rng.choice([1, 33, 70, 256, 300]))
+        while B * S * H * max(D * Cc, T * Cc) > 40_000_000:
+            S = max(1, S // 2)
+        bits = int(rng.choice([10, 20, 30, 40, 63]))
+        rescale = int(rng.choice([0, 19, 21, 23, 29, 37]))
+        q = rand_i64(rng, (B, S, H, D), bits)
+        w1 = rand_i32(rng, (H, D, Cc), int(rng.choice([8, 25, 31])))
+        a = rand_i64(rng, (B, S, H, Cc), bits)
+        kv = rand_i64(rng, (B, T, Cc), int(rng.choice([10, 24, 40])))
+        pr = rand_i64(rng, (B, S, H, T), int(rng.choice([19, 30])))
+        tag = "B=%d S=%d H=%d D=%d C=%d T=%d bits=%d rescale=%d" % (B, S, H, D, Cc, T, bits, rescale)
+        assert np.array_equal(host(K.einsum_bshd_hdc_bshc(dev(q), dev(w1), rescale)), oracle.einsum_bshd_hdc_bshc(q, w1, rescale)), tag
+        assert np.array_equal(host(K.einsum_bshc_btc_bsht(dev(a), dev(kv), rescale)), oracle.einsum_bshc_btc_bsht(a, kv, rescale)), tag
+        assert np.array_equal(host(K.einsum_bsht_btc_bshc(dev(pr), dev(kv), rescale)), oracle.einsum_bsht_btc_bshc(pr, kv, rescale)), tag
+        assert np.array_equal(host(K.einsum_bshc_hdc_bshd(dev(a), dev(w1), rescale)), oracle.einsum_bshc_hdc_bshd(a, w1, rescale)), tag
+
+
 # ---------------------------------------------------------------------------------- einsums -----
 @pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("bits", [20, 40, 63])
