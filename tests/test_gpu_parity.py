@@ -918,3 +918,34 @@ def test_bf16_checkpoint_quantisation(K, oracle):
     assert K.lib.zk_last_error() == 1
     K.lib.zk_clear_error()
 
+
+@pytest.mark.parametrize("seed", range(10))
+def test_rowwise_kernels_seeded_random_problems(K, oracle, seed):
+    """softmax, activations and RMSNorm on random row lengths, row counts, magnitudes and weight types"""
+    rng = np.random.default_rng(9800 + seed)
+    for _ in range(4):
+        T = int(rng.integers(1, 6000))
+        rows = int(rng.integers(1, 40))
+        fn, Q = [("softmax_q19", 19), ("softmax_q21", 21)][int(rng.integers(0, 2))]
+        x = _scores(rng, (1, rows, 1, T), Q)
+        if rng.integers(0, 2):
+            x[0, :, 0, T // 2:] += -(64 << 36)                   # a masked tail
+        R, C = dev(x), torch.empty((1, rows, 1, T), dtype=torch.int64, device="cuda")
+        getattr(K, fn)(R, C)
+        assert np.array_equal(host(C), getattr(oracle, fn)(x)[0]), "%s T=%d rows=%d" % (fn, T, rows)
+        fn, Q = ACTS[int(rng.integers(0, 4))]
+        shape = (1, int(rng.integers(1, 50)), int(rng.integers(1, 5000)))
+        span = int(rng.choice([1, 8, 27, 70]))
+        a = rng.integers(-(span << Q), span << Q, size=shape, dtype=np.int64)
+        R, C = dev(a), torch.empty(shape, dtype=torch.int64, device="cuda")
+        getattr(K, fn)(R, C)
+        assert np.array_equal(host(C), getattr(oracle, fn)(a)), "%s shape=%s span=%d" % (fn, shape, span)
+        N = int(rng.integers(1, 20001))
+        M = int(rng.integers(1, 6))
+        bits = int(rng.choice([8, 20, 31, 37, 50, 63]))
+        A = rand_i64(rng, (M, N), bits)
+        W = rng.integers(1, 1 << 20, size=(N,), dtype=np.int32) if rng.integers(0, 2) else rand_i64(rng, (N,), int(rng.choice([10, 40, 62])))
+        Cn, rms = K.RMS_Norm_int64(dev(A), dev(W), 1, N)
+        Ce, rmse = oracle.RMS_Norm_int64(A, W, 1, N)
+        assert np.array_equal(rms[:M].numpy(), rmse) and np.array_equal(host(Cn), Ce), "rmsnorm M=%d N=%d bits=%d %s" % (M, N, bits, W.dtype)
+
