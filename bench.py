@@ -358,6 +358,24 @@ def main():
         extra["gemm_config2_w2_128x2048x7168"] = gemm_leg(K, H2, W22, 16, 50, 5)
         del X2, W21, H2, W22
 
+        # one token (a decoding step, and the head on every pass): weight streams, reported by the bytes of W per second
+        gd = torch.Generator(device="cuda").manual_seed(1100)
+
+        def gemv_leg(name, Kd, N, w32, b_rs, bits_w):
+            Ad = torch.randint(-(1 << 37), 1 << 37, (1, 1, Kd), generator=gd, dtype=torch.int64, device="cuda")
+            Wd = torch.randint(-(1 << bits_w), 1 << bits_w, (N, Kd), generator=gd, dtype=torch.int64, device="cuda")
+            if w32:
+                Wd = Wd.to(torch.int32)
+            Cd = torch.empty((1, 1, N), dtype=torch.int64, device="cuda")
+            fn = K.lib.int64_32_bmm_broadcast_launcher if w32 else K.lib.int64_64_bmm_broadcast_launcher
+            call = lambda: fn(Ad.data_ptr(), Wd.data_ptr(), Cd.data_ptr(), None, 1, b_rs, 29, 1, 1, Kd, N)
+            hbm(name, call, N * Kd, bytes_per_elem=4.0 if w32 else 8.0, steps=20)
+            extra[name]["path"] = {1: "valu", 2: "mfma_i8"}.get(K.gemm_last_plan()[0], "?")
+
+        gemv_leg("gemm_1token_head_7168x129280_int64_div256", 7168, 129280, False, 256, 43)
+        gemv_leg("gemm_1token_wo_16384x7168_int32", 16384, 7168, True, 1, 31)
+        gemv_leg("gemm_1token_wkv_a_7168x576_int32", 7168, 576, True, 1, 31)
+
         # the four MLA einsums at config 3's shape (S = T = 1024, 128 heads, absorb mode: model.py:884-936), Q30
         # activations against Q24 cache entries / int32 Q25 weights
         ge = torch.Generator(device="cuda").manual_seed(900)

@@ -30,6 +30,10 @@ enum GemmPath { kPathAuto = 0, kPathValu = 1, kPathMfma = 2 };
 // pointer) the launch is conditional: its workgroups return at once unless *guard is non-zero when they start.
 void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard = nullptr);
 
+// Matrix-vector kernel of the same family for one or two rows of A against k-contiguous B: one launch, nothing
+// guessed.  Returns false (nothing launched) for any other descriptor.
+bool gemm_gemv_launch(const GemmDesc &d);
+
 // Limb-decomposed i8 MFMA.  Returns false (nothing launched) when the descriptor is outside what it
 // supports, in which case the caller falls back to the VALU path.
 bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);

@@ -13,6 +13,13 @@ static long g_grouped_mfma_calls = 0;
 
 void gemm_dispatch(const char *name, const GemmDesc &d)
 {
+    // one or two rows (a decoding step, the head): the exact vector-ALU stream over the weights, unless the MFMA
+    // path is asked for by name
+    if (g_gemm_path != kPathMfma && gemm_gemv_launch(d)) {
+        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+        check_launch(name);
+        return;
+    }
     if (g_gemm_path != kPathValu) {
         int la = 0, lb = 0;
         if (gemm_mfma_launch(d, &la, &lb)) {

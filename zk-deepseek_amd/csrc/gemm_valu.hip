@@ -9,6 +9,8 @@
 // The same kernel is the safety net of the speculating MFMA path: launched with a `guard` word, its workgroups
 // return at once unless that word says the speculation failed, in which case they recompute every output.
 #include "gemm.h"
+#include <type_traits>
+#include <cstdlib>
 
 namespace zk {
 
@@ -164,6 +166,214 @@ void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard)
     dim3 grid((unsigned)(p.tiles < cap ? p.tiles : cap));
     if (d.b32) { if (kmajor) launch2<true, true>(p, grid, rescale); else launch2<true, false>(p, grid, rescale); }
     else { if (kmajor) launch2<false, true>(p, grid, rescale); else launch2<false, false>(p, grid, rescale); }
+}
+
+// ---- one or two rows of A: a matrix-vector product -----------------------------------------------------------
+// Decoding runs every projection, and the head always, on a single token (inference/model.py:1519, 1599-1606): the
+// product is a stream over the weights with next to no reuse, and exact 128-bit multiply-adds on the vector ALU keep
+// up with that stream, so nothing has to be guessed about the operands and one launch does it all.
+// A wave takes COLS columns of the output (rows of B) at a time (four once there are columns enough to fill the device
+// that way, so that every element of A it loads meets four weights; else one); WPC waves share such a group, each
+// taking every WPC-th stretch of K, and a workgroup of four waves covers 4 / WPC groups.  A lane loads 16 bytes of a B
+// row at a time (two int64 or four int32 weights) and the matching elements of each A row, 4-8 such loads per row in
+// flight, and keeps one 128-bit sum per output.  Bytes in flight are what this kernel lives on: with 8-byte loads of
+// int32 weights it streamed 1.7 TB/s, with 16-byte loads 3.4 TB/s.
+constexpr int kGemvMaxM = 2;
+
+// A 128-bit sum kept as a 64-bit low word and a count of what went past it, so that adding a signed 64-bit product is
+// four independent-looking instructions (sign word, add, add-with-carry twice) instead of a four-word carry chain.
+struct SplitSum {
+    uint64_t lo = 0;
+    int32_t over = 0;                      // carries out of lo minus the negative addends: the sum is lo + 2^64 * over
+    __device__ __forceinline__ void add(int64_t x)
+    {
+        const uint64_t t = lo + (uint64_t)x;
+        over += (int32_t)(t < lo) + (int32_t)(x >> 63);
+        lo = t;
+    }
+    __device__ __forceinline__ u128 total() const { return (u128)lo + ((u128)(i128)(int64_t)over << 64); }
+};
+
+template <bool B32, bool RESCALE, int MR, int WPC, int COLS>
+__global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
+{
+    constexpr int UN = COLS == 1 ? (B32 ? 4 : 8) : (B32 ? 2 : 4);       // 16-byte loads per B row in flight
+    __shared__ u128 part[4][COLS][MR];
+    typedef typename std::conditional<B32, int32_t, int64_t>::type BT;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int group = wave / WPC, slice = wave % WPC;
+    const long n0 = ((long)blockIdx.x * (4 / WPC) + group) * COLS;
+    const int g = blockIdx.y;
+    const int64_t *Ag = p.A + (long)g * p.sA;
+    long brow[COLS];                                   // columns past N read the last row; their sums are dropped
+#pragma unroll
+    for (int c = 0; c < COLS; c++) brow[c] = (long)g * p.sB + (n0 + c < p.N ? n0 + c : p.N - 1) * p.ldbn;
+    u128 acc[COLS][MR];
+#pragma unroll
+    for (int c = 0; c < COLS; c++)
+#pragma unroll
+        for (int m = 0; m < MR; m++) acc[c][m] = 0;
+
+    // int32 weights without divisors: a = ah * 2^32 + al (ah signed, al unsigned) meets b in two 64-bit products, a
+    // third of the multiplies of the general case, and each kind has its own split sum (weights 2^32 and 1)
+    constexpr bool SPLIT = B32 && !RESCALE;
+    SplitSum shi[SPLIT ? COLS : 1][SPLIT ? MR : 1], slo[SPLIT ? COLS : 1][SPLIT ? MR : 1];
+    auto mac = [&](int c, int m, int64_t a, int64_t b) {
+        if (SPLIT) {
+            const int32_t b32 = (int32_t)b;
+            shi[c][m].add((int64_t)(int32_t)(a >> 32) * (int64_t)b32);
+            slo[c][m].add((int64_t)(uint64_t)(uint32_t)a * (int64_t)b32);            // |al * b| < 2^63
+        } else {
+            if (RESCALE) { a = rescale_operand(a, p.a_rs, p.a_shift); b = rescale_operand(b, p.b_rs, p.b_shift); }
+            acc[c][m] += (u128)((i128)a * (i128)b);
+        }
+    };
+    // units of EPL consecutive k (16 bytes of a B row): every pointer and stride keeps the 16-byte loads aligned
+    // (decided on the host)
+    constexpr int EPL = B32 ? 4 : 2;
+    const int units = p.tiles_m ? p.K / EPL : 0;       // tiles_m doubles as the "vector loads allowed" flag here
+    if (n0 < p.N) {
+        for (int q0 = slice * 64 * UN; q0 < units; q0 += WPC * 64 * UN) {
+            BT b[UN][COLS][EPL];
+            int64_t a[UN][MR][EPL];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int q = q0 + u * 64 + lane;
+                const bool in = q < units;
+#pragma unroll
+                for (int c = 0; c < COLS; c++) {
+#pragma unroll
+                    for (int e = 0; e < EPL; e++) b[u][c][e] = 0;
+                    if (in) {
+                        if (B32) {
+                            const int4 t = *reinterpret_cast<const int4 *>(reinterpret_cast<const int32_t *>(p.B) + brow[c] + 4 * q);
+                            b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y; b[u][c][2 % EPL] = (BT)t.z; b[u][c][3 % EPL] = (BT)t.w;
+                        } else {
+                            const longlong2 t = *reinterpret_cast<const longlong2 *>(reinterpret_cast<const int64_t *>(p.B) + brow[c] + 2 * q);
+                            b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MR; m++)
+#pragma unroll
+                    for (int h = 0; h < EPL / 2; h++) {
+                        a[u][m][2 * h] = a[u][m][2 * h + 1] = 0;
+                        if (in) {
+                            const longlong2 t = *reinterpret_cast<const longlong2 *>(Ag + (long)m * p.lda + (long)EPL * q + 2 * h);
+                            a[u][m][2 * h] = t.x; a[u][m][2 * h + 1] = t.y;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++)
+#pragma unroll
+                for (int c = 0; c < COLS; c++)
+#pragma unroll
+                    for (int m = 0; m < MR; m++)
+#pragma unroll
+                        for (int e = 0; e < EPL; e++) mac(c, m, a[u][m][e], b[u][c][e]);
+        }
+        // what the units left over (all of K when vector loads are not allowed)
+        for (int k = EPL * units + slice * 64 + lane; k < p.K; k += WPC * 64) {
+#pragma unroll
+            for (int c = 0; c < COLS; c++) {
+                const int64_t bv = load_b<B32>(p.B, brow[c] + k);
+#pragma unroll
+                for (int m = 0; m < MR; m++) mac(c, m, Ag[(long)m * p.lda + k], bv);
+            }
+        }
+    }
+
+    // lanes, then the waves of a group
+#pragma unroll
+    for (int c = 0; c < COLS; c++)
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            if (SPLIT) acc[c][m] = (shi[c][m].total() << 32) + slo[c][m].total();
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const uint64_t lo = (uint64_t)__shfl_xor((long long)(uint64_t)acc[c][m], off, 64);
+                const uint64_t hi = (uint64_t)__shfl_xor((long long)(uint64_t)(acc[c][m] >> 64), off, 64);
+                acc[c][m] += ((u128)hi << 64) | lo;
+            }
+        }
+    if (WPC > 1) {
+        if (lane == 0)
+#pragma unroll
+            for (int c = 0; c < COLS; c++)
+#pragma unroll
+                for (int m = 0; m < MR; m++) part[wave][c][m] = acc[c][m];
+        __syncthreads();
+        if (slice != 0) return;
+#pragma unroll
+        for (int c = 0; c < COLS; c++)
+#pragma unroll
+            for (int m = 0; m < MR; m++)
+#pragma unroll
+                for (int w = 1; w < WPC; w++) acc[c][m] += part[group * WPC + w][c][m];
+    }
+    if (lane != 0) return;
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+#pragma unroll
+    for (int c = 0; c < COLS; c++) {
+        if (n0 + c >= p.N) break;
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            if (m >= p.M) break;
+            const u128 sum = acc[c][m] + (u128)(i128)p.init;
+            const long o = (long)g * p.sC + (long)m * p.ldc + n0 + c;
+            p.C[o] = (int64_t)(uint64_t)((i128)sum >> p.shift);
+            if (p.R) p.R[o] = (int64_t)((uint64_t)sum & rmask);
+        }
+    }
+}
+
+template <bool B32, bool RESCALE, int MR, int COLS>
+static void gemv_launch4(const ValuParams &p, int G)
+{
+    // enough waves to keep the weight stream busy: four per column group for a narrow output, one for a wide one
+    const long groups = (p.N + COLS - 1) / COLS, waves1 = groups * G;
+    if (waves1 >= 8192) gemv_kernel<B32, RESCALE, MR, 1, COLS><<<dim3((unsigned)((groups + 3) / 4), (unsigned)G), dim3(256), 0, 0>>>(p);
+    else if (waves1 >= 4096) gemv_kernel<B32, RESCALE, MR, 2, COLS><<<dim3((unsigned)((groups + 1) / 2), (unsigned)G), dim3(256), 0, 0>>>(p);
+    else gemv_kernel<B32, RESCALE, MR, 4, COLS><<<dim3((unsigned)groups, (unsigned)G), dim3(256), 0, 0>>>(p);
+}
+
+template <bool B32, bool RESCALE, int MR>
+static void gemv_launch3(const ValuParams &p, int G)
+{
+    // four columns per wave share each load of A, once there are columns enough to fill the device that way
+    if ((long)p.N * G >= 4 * 8192) gemv_launch4<B32, RESCALE, MR, 4>(p, G);
+    else gemv_launch4<B32, RESCALE, MR, 1>(p, G);
+}
+
+bool gemm_gemv_launch(const GemmDesc &d)
+{
+    if (d.M < 1 || d.M > kGemvMaxM || d.ldbk != 1 || d.G > 65535 || d.N < 1 || d.K < 1) return false;
+    ValuParams p = {};
+    p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
+    p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
+    p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift;
+    p.init = d.init; p.a_rs = d.a_rs; p.b_rs = d.b_rs;
+    auto log2_exact = [](int64_t v) {
+        if (v <= 0 || (v & (v - 1)) != 0) return -1;
+        int s = 0;
+        while (((int64_t)1 << s) < v) s++;
+        return s;
+    };
+    p.a_shift = log2_exact(d.a_rs);
+    p.b_shift = log2_exact(d.b_rs);
+    // the 16-byte loads need 16-byte aligned rows of A and of B
+    const size_t esz = d.b32 ? 4 : 8;
+    const bool a_ok = (((uintptr_t)d.A | (uintptr_t)(d.lda * 8) | (uintptr_t)(d.sA * 8)) & 15) == 0;
+    const bool b_ok = (((uintptr_t)d.B | (uintptr_t)(d.ldbn * esz) | (uintptr_t)(d.sB * esz)) & 15) == 0;
+    p.tiles_m = (a_ok && b_ok) ? 1 : 0;
+    const bool rescale = d.a_rs != 1 || d.b_rs != 1;
+#define ZK_GEMV(B32, RS) do { if (d.M == 1) gemv_launch3<B32, RS, 1>(p, d.G); else gemv_launch3<B32, RS, 2>(p, d.G); } while (0)
+    if (d.b32) { if (rescale) ZK_GEMV(true, true); else ZK_GEMV(true, false); }
+    else { if (rescale) ZK_GEMV(false, true); else ZK_GEMV(false, false); }
+#undef ZK_GEMV
+    return true;
 }
 
 }  // namespace zk
