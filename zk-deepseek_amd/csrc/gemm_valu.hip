@@ -10,7 +10,6 @@
 // return at once unless that word says the speculation failed, in which case they recompute every output.
 #include "gemm.h"
 #include <type_traits>
-#include <cstdlib>
 
 namespace zk {
 
@@ -172,12 +171,11 @@ void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard)
 // Decoding runs every projection, and the head always, on a single token (inference/model.py:1519, 1599-1606): the
 // product is a stream over the weights with next to no reuse, and exact 128-bit multiply-adds on the vector ALU keep
 // up with that stream, so nothing has to be guessed about the operands and one launch does it all.
-// A wave takes COLS columns of the output (rows of B) at a time (four once there are columns enough to fill the device
-// that way, so that every element of A it loads meets four weights; else one); WPC waves share such a group, each
-// taking every WPC-th stretch of K, and a workgroup of four waves covers 4 / WPC groups.  A lane loads 16 bytes of a B
-// row at a time (two int64 or four int32 weights) and the matching elements of each A row, 4-8 such loads per row in
-// flight, and keeps one 128-bit sum per output.  Bytes in flight are what this kernel lives on: with 8-byte loads of
-// int32 weights it streamed 1.7 TB/s, with 16-byte loads 3.4 TB/s.
+// A wave takes one column of the output (a row of B); WPC waves share it, each taking every WPC-th stretch of K, and
+// a workgroup of four waves covers 4 / WPC columns.  A lane loads 16 bytes of the B row at a time (two int64 or four
+// int32 weights) and the matching elements of each A row, 4-8 such loads in flight, and keeps one 128-bit sum per
+// output.  Bytes in flight are what this kernel lives on: with 8-byte loads of int32 weights it streamed 1.7 TB/s,
+// with 16-byte loads 3.4 TB/s.
 constexpr int kGemvMaxM = 2;
 
 // A 128-bit sum kept as a 64-bit low word and a count of what went past it, so that adding a signed 64-bit product is
@@ -194,10 +192,13 @@ struct SplitSum {
     __device__ __forceinline__ u128 total() const { return (u128)lo + ((u128)(i128)(int64_t)over << 64); }
 };
 
-template <bool B32, bool RESCALE, int MR, int WPC, int COLS>
+template <bool B32, bool RESCALE, int MR, int WPC>
 __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
 {
-    constexpr int UN = COLS == 1 ? (B32 ? 4 : 8) : (B32 ? 2 : 4);       // 16-byte loads per B row in flight
+    // One column per wave: several columns per wave would share the loads of A, and measured slower at every size
+    // (the head: 1.33 ms with four against 1.27 ms), so COLS stays a constant of the code rather than a choice.
+    constexpr int COLS = 1;
+    constexpr int UN = B32 ? 4 : 8;                    // 16-byte loads per B row in flight
     __shared__ u128 part[4][COLS][MR];
     typedef typename std::conditional<B32, int32_t, int64_t>::type BT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -329,22 +330,14 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
     }
 }
 
-template <bool B32, bool RESCALE, int MR, int COLS>
-static void gemv_launch4(const ValuParams &p, int G)
-{
-    // enough waves to keep the weight stream busy: four per column group for a narrow output, one for a wide one
-    const long groups = (p.N + COLS - 1) / COLS, waves1 = groups * G;
-    if (waves1 >= 8192) gemv_kernel<B32, RESCALE, MR, 1, COLS><<<dim3((unsigned)((groups + 3) / 4), (unsigned)G), dim3(256), 0, 0>>>(p);
-    else if (waves1 >= 4096) gemv_kernel<B32, RESCALE, MR, 2, COLS><<<dim3((unsigned)((groups + 1) / 2), (unsigned)G), dim3(256), 0, 0>>>(p);
-    else gemv_kernel<B32, RESCALE, MR, 4, COLS><<<dim3((unsigned)groups, (unsigned)G), dim3(256), 0, 0>>>(p);
-}
-
 template <bool B32, bool RESCALE, int MR>
 static void gemv_launch3(const ValuParams &p, int G)
 {
-    // four columns per wave share each load of A, once there are columns enough to fill the device that way
-    if ((long)p.N * G >= 4 * 8192) gemv_launch4<B32, RESCALE, MR, 4>(p, G);
-    else gemv_launch4<B32, RESCALE, MR, 1>(p, G);
+    // enough waves to keep the weight stream busy: four per column for a narrow output, one for a wide one
+    const long waves1 = (long)p.N * G;
+    if (waves1 >= 8192) gemv_kernel<B32, RESCALE, MR, 1><<<dim3((unsigned)((p.N + 3) / 4), (unsigned)G), dim3(256), 0, 0>>>(p);
+    else if (waves1 >= 4096) gemv_kernel<B32, RESCALE, MR, 2><<<dim3((unsigned)((p.N + 1) / 2), (unsigned)G), dim3(256), 0, 0>>>(p);
+    else gemv_kernel<B32, RESCALE, MR, 4><<<dim3((unsigned)p.N, (unsigned)G), dim3(256), 0, 0>>>(p);
 }
 
 bool gemm_gemv_launch(const GemmDesc &d)
