@@ -180,6 +180,14 @@ def test_gemm_one_or_two_rows(K, oracle, M, w32):
     A, W = rand_i64(rng, (1, M, 300), 45), (rand_i32(rng, (77, 300)) if w32 else rand_i64(rng, (77, 300), 50))
     for a_rs, b_rs in ((1, 256), (3, 1), (-7, 5), (1 << 20, 1 << 3)):
         _gemm_case(K, oracle, 0, A, W, a_rs, b_rs, 21)
+    # the per-head einsums of a decoding step: M rows per head, the heads as a strided batch
+    H, D, Cc = 16, 24, 40
+    a = rand_i64(rng, (1, M, H, Cc), 30)
+    w = rand_i32(rng, (H, D, Cc), 25)
+    assert np.array_equal(host(K.einsum_bshc_hdc_bshd(dev(a), dev(w), 21)), oracle.einsum_bshc_hdc_bshd(a, w, 21))
+    assert K.gemm_last_plan()[0] == 1
+    q = rand_i64(rng, (1, M, H, D), 30)
+    assert np.array_equal(host(K.einsum_bshd_hdc_bshc(dev(q), dev(w), 21)), oracle.einsum_bshd_hdc_bshc(q, w, 21))
     # rows of A that start 8 bytes off a 16-byte boundary: the element-wise loads
     buf = torch.zeros((M * 301 + 1,), dtype=torch.int64, device="cuda")
     Av = rand_i64(rng, (1, M, 301), 40)
