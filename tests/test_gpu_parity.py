@@ -188,6 +188,7 @@ def test_gemm_one_or_two_rows(K, oracle, M, w32):
     assert K.gemm_last_plan()[0] == 1
     q = rand_i64(rng, (1, M, H, D), 30)
     assert np.array_equal(host(K.einsum_bshd_hdc_bshc(dev(q), dev(w), 21)), oracle.einsum_bshd_hdc_bshc(q, w, 21))
+    assert K.gemm_last_plan()[0] == 1
     # rows of A that start 8 bytes off a 16-byte boundary: the element-wise loads
     buf = torch.zeros((M * 301 + 1,), dtype=torch.int64, device="cuda")
     Av = rand_i64(rng, (1, M, 301), 40)

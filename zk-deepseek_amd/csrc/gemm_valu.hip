@@ -330,6 +330,41 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
     }
 }
 
+// The same for n-contiguous B (the per-head weights of `bshd,hdc->bshc`): a lane owns an output column and walks K, the
+// loads of a row of B are contiguous over the wave, and the elements of A are the same for every lane.
+template <bool B32, bool RESCALE, int MR>
+__global__ __launch_bounds__(256) void gemv_kmajor_kernel(ValuParams p)
+{
+    const long n = (long)blockIdx.x * 256 + threadIdx.x;
+    const int g = blockIdx.y;
+    if (n >= p.N) return;
+    const int64_t *Ag = p.A + (long)g * p.sA;
+    const long b0 = (long)g * p.sB + n;
+    u128 acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) acc[m] = 0;
+#pragma unroll 4
+    for (int k = 0; k < p.K; k++) {
+        int64_t b = load_b<B32>(p.B, b0 + (long)k * p.ldbk);
+        if (RESCALE) b = rescale_operand(b, p.b_rs, p.b_shift);
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            int64_t a = Ag[(long)m * p.lda + k];
+            if (RESCALE) a = rescale_operand(a, p.a_rs, p.a_shift);
+            acc[m] += (u128)((i128)a * (i128)b);
+        }
+    }
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+#pragma unroll
+    for (int m = 0; m < MR; m++) {
+        if (m >= p.M) break;
+        const u128 sum = acc[m] + (u128)(i128)p.init;
+        const long o = (long)g * p.sC + (long)m * p.ldc + n;
+        p.C[o] = (int64_t)(uint64_t)((i128)sum >> p.shift);
+        if (p.R) p.R[o] = (int64_t)((uint64_t)sum & rmask);
+    }
+}
+
 template <bool B32, bool RESCALE, int MR>
 static void gemv_launch3(const ValuParams &p, int G)
 {
@@ -342,7 +377,11 @@ static void gemv_launch3(const ValuParams &p, int G)
 
 bool gemm_gemv_launch(const GemmDesc &d)
 {
-    if (d.M < 1 || d.M > kGemvMaxM || d.ldbk != 1 || d.G > 65535 || d.N < 1 || d.K < 1) return false;
+    if (d.M < 1 || d.M > kGemvMaxM || d.G > 65535 || d.N < 1 || d.K < 1) return false;
+    const bool kmajor = d.ldbn == 1 && d.ldbk != 1;
+    if (!kmajor && d.ldbk != 1) return false;
+    // an n-contiguous B is walked by one thread per column: fine for the short K of the einsum that has it, not for more
+    if (kmajor && d.K > 1024) return false;
     ValuParams p = {};
     p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
     p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
@@ -362,6 +401,15 @@ bool gemm_gemv_launch(const GemmDesc &d)
     const bool b_ok = (((uintptr_t)d.B | (uintptr_t)(d.ldbn * esz) | (uintptr_t)(d.sB * esz)) & 15) == 0;
     p.tiles_m = (a_ok && b_ok) ? 1 : 0;
     const bool rescale = d.a_rs != 1 || d.b_rs != 1;
+    if (kmajor) {
+        const dim3 grid((unsigned)((d.N + 255) / 256), (unsigned)d.G);
+#define ZK_GEMVK(B32, RS) do { if (d.M == 1) gemv_kmajor_kernel<B32, RS, 1><<<grid, dim3(256), 0, 0>>>(p); \
+                               else gemv_kmajor_kernel<B32, RS, 2><<<grid, dim3(256), 0, 0>>>(p); } while (0)
+        if (d.b32) { if (rescale) ZK_GEMVK(true, true); else ZK_GEMVK(true, false); }
+        else { if (rescale) ZK_GEMVK(false, true); else ZK_GEMVK(false, false); }
+#undef ZK_GEMVK
+        return true;
+    }
 #define ZK_GEMV(B32, RS) do { if (d.M == 1) gemv_launch3<B32, RS, 1>(p, d.G); else gemv_launch3<B32, RS, 2>(p, d.G); } while (0)
     if (d.b32) { if (rescale) ZK_GEMV(true, true); else ZK_GEMV(true, false); }
     else { if (rescale) ZK_GEMV(false, true); else ZK_GEMV(false, false); }
