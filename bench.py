@@ -315,6 +315,24 @@ def main():
             extra["moe_experts_config5_256tok_top8_of_256"]["weight_bytes"] = wbytes
             del ew1, ew3, ew2, tabs
             torch.cuda.empty_cache()
+            # the same with the model's weight type: int32 at 31 bits (45 GB), shifts that keep the activations in Q23
+            # range; 256 tokens (three grouped MFMA launches) and one token (three grouped matrix-vector launches)
+            mk32 = lambda *shape: torch.randint(-(1 << 30), 1 << 30, shape, generator=gm, dtype=torch.int64, device="cuda").to(torch.int32)
+            ew1 = [mk32(2048, 7168) for _ in range(256)]
+            ew3 = [mk32(2048, 7168) for _ in range(256)]
+            ew2 = [mk32(7168, 2048) for _ in range(256)]
+            tabs = [K.pointer_table(w) for w in (ew1, ew3, ew2)]
+            for Tt in (256, 1):
+                wt, it = wm[:Tt].contiguous(), im[:Tt].contiguous()
+                xt = xm[:Tt].contiguous()
+                hit = int(torch.unique(it).numel())
+                wbytes = 3.0 * hit * 2048 * 7168 * 4
+                nm = "moe_experts_int32_%dtok_top8_of_256" % Tt
+                hbm(nm, lambda: K.moe_experts(xt, wt, it, tabs[0], tabs[1], tabs[2], True, 2048, 30, 33), 1, bytes_per_elem=wbytes, steps=3)
+                extra[nm]["weight_bytes"] = wbytes
+                extra[nm]["experts_hit"] = hit
+            del ew1, ew3, ew2, tabs
+            torch.cuda.empty_cache()
 
         # witness dump: what one layer's ~30 saveTensor calls cost the host thread, against the reference's way
         # (synchronous .cpu() + tobytes + write, inference/model.py:94-102); files go to a temporary directory

@@ -859,6 +859,30 @@ def test_int64_grouped_bmm(K, oracle, path, w32, bits):
 
 
 @pytest.mark.parametrize("w32", [False, True])
+@pytest.mark.parametrize("T,Kr,Kd,N", [(1, 8, 520, 300), (2, 8, 7168, 64), (4, 3, 333, 1030), (1, 1, 64, 5000)])
+def test_int64_grouped_bmm_few_rows(K, oracle, w32, T, Kr, Kd, N):
+    """a decoding step's routed experts: up to 32 rows go row by row through the matrix-vector kernel in one launch
+    (every row against the weights of its own expert, empty experts in between, odd K, the remainder output)"""
+    rng = np.random.default_rng(T * 100 + Kr + w32)
+    E = 16
+    idx = _routing(rng, T, E, Kr)
+    x = rand_i64(rng, (T, Kd), 40)
+    ws = [rand_i32(rng, (N, Kd), 31) if w32 else rand_i64(rng, (N, Kd), 50) for _ in range(E)]
+    K.lib.zk_gemm_set_path(0)
+    d = K.moe_dispatch(dev(idx), E)
+    xs = K.moe_gather_rows(dev(x), d)
+    seg, tok, _ = oracle.moe_dispatch(idx, E)
+    wd = [dev(w) for w in ws]
+    before = K.lib.zk_gemm_grouped_mfma_calls()
+    for c in (0, 23):
+        C, R = K.int64_grouped_bmm(xs, K.pointer_table(wd), w32, N, c, d, want_remainder=True)
+        Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
+        assert np.array_equal(host(C), Ce), "quotient"
+        assert np.array_equal(host(R), Re), "remainder"
+    assert K.lib.zk_gemm_grouped_mfma_calls() == before and K.gemm_last_plan()[0] == 1
+
+
+@pytest.mark.parametrize("w32", [False, True])
 def test_moe_experts(K, oracle, w32):
     """routed experts end to end (dispatch, gather, grouped gate/up GEMMs, SiLU gate, grouped down GEMM, weighted
     combine) against the reference's loop over the experts restated on the oracle"""

@@ -61,6 +61,11 @@ struct GroupedDesc {
     int64_t init;
 };
 
+// The grouped product row by row on the matrix-vector kernel: one launch, every row of A against the B of its segment.
+// Streams a B once per row of its segment, so it is for a handful of rows (a decoding step's routed experts).
+// Returns false (nothing launched) when the descriptor is outside what it takes.
+bool gemm_gemv_grouped_launch(const GroupedDesc &d);
+
 // One launch of the 32-row-tile MFMA kernels over all groups.  Returns 0 when done, 1 when the operands need
 // more digits than those kernels are built for (nothing valid was written: the caller takes another route),
 // -1 on an error (recorded).

@@ -914,7 +914,10 @@ struct Instance {
 };
 
 
-template <int NA, int NB, bool SKINNY = false, int DMAX = 16>
+// KKSEL: MFMA k-depths (of 32) per pipeline step.  B32ONLY: an instance for int32 B alone.  The 32-row kernels live on
+// the bytes they keep in flight, and a step of int32 weights is half the bytes of a step of int64 weights: with two
+// depths per step they stream as much per step as the int64 kernels do (where the two LDS stages still fit).
+template <int NA, int NB, bool SKINNY = false, int DMAX = 16, int KKSEL = ZK_KK(0), bool B32ONLY = false>
 static Instance make_instance()
 {
     constexpr int DD = (NA + NB - 1) > DMAX ? DMAX : (NA + NB - 1);      // diagonals kept = accumulator sets
@@ -925,25 +928,28 @@ static Instance make_instance()
     constexpr int WVM = SKINNY ? 1 : (DD <= 5 ? 2 : (DD <= 10 ? 4 : 2));
     constexpr int WVN = SKINNY ? 8 : (DD <= 5 ? 4 : 2);
     constexpr int WM = SKINNY ? 1 : (DD <= 5 ? 2 : 1), WN = 1;
-    constexpr int KK = ZK_KK(DD);
+    constexpr int KK = KKSEL;
+    static_assert(!B32ONLY || NB <= 5, "int32 values never need more than five digits");
     Instance s;
     s.na = NA; s.nb = NB; s.bm = 32 * WM * WVM; s.bn = 32 * WN * WVN; s.threads = 64 * WVM * WVN; s.kk = KK;
     s.skinny = SKINNY;
     s.dmax = DMAX;
     for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
-    s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, false, DMAX>;
-    s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX>;
-    s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false, false, false, DMAX>;
+    if constexpr (!B32ONLY) {
+        s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, false, DMAX>;
+        s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX>;
+        s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false, false, false, DMAX>;
+    }
     if constexpr (NB <= 5) {          // int32 values never need more than five digits
         s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, false, DMAX>;
         s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true, false, false, DMAX>;
         s.fn[kB32KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, true, false, false, false, DMAX>;
     }
     if constexpr (SKINNY) {          // grouped launches (one B per segment of rows) run on the 32-row tiles only
-        s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX>;
+        if constexpr (!B32ONLY) s.fn[kB64Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX>;
         if constexpr (NB <= 5) s.fn[kB32Group] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, true, false, DMAX>;
         // and so do products whose B is divided by a power of two first (the model's head projection)
-        s.fn[kB64FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, true, DMAX>;
+        if constexpr (!B32ONLY) s.fn[kB64FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, true, DMAX>;
         if constexpr (NB <= 5) s.fn[kB32FlyRs] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, true, DMAX>;
     }
     s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
@@ -963,6 +969,9 @@ static const Instance *instances(int *count)
         make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(),
         make_instance<9, 5>(), make_instance<5, 9>(), make_instance<9, 9>(),
         make_instance<3, 3, true>(), make_instance<5, 5, true>(),
+        // 28-bit activations against 31-bit weights: what an expert sees after the norm (inference/model.py:1017, 1324)
+        make_instance<4, 4, true>(), make_instance<4, 5, true>(),
+        make_instance<3, 3, true, 16, 2, true>(), make_instance<4, 4, true, 16, 2, true>(),
         // many-digit operands whose shift + 64 result bits end below 2^96 or 2^64: fewer digit pairs
         make_instance<9, 9, false, 12>(), make_instance<9, 9, false, 8>(),
         make_instance<9, 5, false, 8>(), make_instance<5, 9, false, 8>(),
@@ -983,8 +992,10 @@ static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int 
         if (t[i].na < na || t[i].nb < nb || t[i].skinny != skinny) continue;
         if (t[i].dmax < 16 && t[i].dmax < need_diag) continue;
         if (b32 && !t[i].fn[kB32Fly]) continue;
+        if (!b32 && !t[i].fn[kB64Fly]) continue;
         long cost = kept_pairs_before(t[i].na, t[i].nb, t[i].dmax, t[i].na, 0);     // MFMAs per 32x32x32 block
-        if (!best || cost < best_cost) { best = &t[i]; best_cost = cost; }
+        // at equal MFMA count the deeper step wins (only instances made for int32 B have one)
+        if (!best || cost < best_cost || (cost == best_cost && t[i].kk > best->kk)) { best = &t[i]; best_cost = cost; }
     }
     return best;
 }
@@ -1338,8 +1349,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
     p.split = 1; p.finish_rq = 4;
     p.grp_seg = d.seg; p.grp_tiles = d.tiles; p.grp_ntiles = d.ntiles; p.grp_b = d.B;
 
-    // digits: what these operands needed last time, else the widest the 32-row kernels have (the launch is bound
-    // by the weight stream, not by the MFMA count)
+    // digits: what these operands needed last time, else the widest the 32-row kernels have
     const OperandKey key_a(d.A, (long)d.rows, d.K, 8), key_b(d.B, (long)d.groups * d.N, d.K, d.b32 ? 4 : 8);
     int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
     if (!na) {

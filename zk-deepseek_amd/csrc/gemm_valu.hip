@@ -28,6 +28,10 @@ struct ValuParams {
     int tiles_m, tiles_n;
     long tiles;                               // tiles_m * tiles_n * G, walked by a 1-D grid
     const unsigned long long *guard;          // when set: do nothing unless *guard != 0
+    // grouped matrix-vector launches: blockIdx.y is a row of A, whose B is that of the segment the row lies in
+    const void *const *grp_b;                 // device array of `groups` device pointers
+    const int *grp_seg;                       // device [groups + 1]: first row of every segment
+    int groups;
 };
 
 template <bool B32>
@@ -192,7 +196,7 @@ struct SplitSum {
     __device__ __forceinline__ u128 total() const { return (u128)lo + ((u128)(i128)(int64_t)over << 64); }
 };
 
-template <bool B32, bool RESCALE, int MR, int WPC>
+template <bool B32, bool RESCALE, int MR, int WPC, bool GRP = false>
 __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
 {
     // One column per wave: several columns per wave would share the loads of A, and measured slower at every size
@@ -206,6 +210,17 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
     const long n0 = ((long)blockIdx.x * (4 / WPC) + group) * COLS;
     const int g = blockIdx.y;
     const int64_t *Ag = p.A + (long)g * p.sA;
+    const void *Bbase = p.B;
+    if (GRP) {
+        // the segment that holds row g: the last one that starts at or before it (empty segments share a start with
+        // their successor and lose to it)
+        int lo = 0, hi = p.groups - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (p.grp_seg[mid] <= g) lo = mid; else hi = mid - 1;
+        }
+        Bbase = p.grp_b[lo];
+    }
     long brow[COLS];                                   // columns past N read the last row; their sums are dropped
 #pragma unroll
     for (int c = 0; c < COLS; c++) brow[c] = (long)g * p.sB + (n0 + c < p.N ? n0 + c : p.N - 1) * p.ldbn;
@@ -247,10 +262,10 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
                     for (int e = 0; e < EPL; e++) b[u][c][e] = 0;
                     if (in) {
                         if (B32) {
-                            const int4 t = *reinterpret_cast<const int4 *>(reinterpret_cast<const int32_t *>(p.B) + brow[c] + 4 * q);
+                            const int4 t = *reinterpret_cast<const int4 *>(reinterpret_cast<const int32_t *>(Bbase) + brow[c] + 4 * q);
                             b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y; b[u][c][2 % EPL] = (BT)t.z; b[u][c][3 % EPL] = (BT)t.w;
                         } else {
-                            const longlong2 t = *reinterpret_cast<const longlong2 *>(reinterpret_cast<const int64_t *>(p.B) + brow[c] + 2 * q);
+                            const longlong2 t = *reinterpret_cast<const longlong2 *>(reinterpret_cast<const int64_t *>(Bbase) + brow[c] + 2 * q);
                             b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y;
                         }
                     }
@@ -279,7 +294,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
         for (int k = EPL * units + slice * 64 + lane; k < p.K; k += WPC * 64) {
 #pragma unroll
             for (int c = 0; c < COLS; c++) {
-                const int64_t bv = load_b<B32>(p.B, brow[c] + k);
+                const int64_t bv = load_b<B32>(Bbase, brow[c] + k);
 #pragma unroll
                 for (int m = 0; m < MR; m++) mac(c, m, Ag[(long)m * p.lda + k], bv);
             }
@@ -373,6 +388,31 @@ static void gemv_launch3(const ValuParams &p, int G)
     if (waves1 >= 8192) gemv_kernel<B32, RESCALE, MR, 1><<<dim3((unsigned)((p.N + 3) / 4), (unsigned)G), dim3(256), 0, 0>>>(p);
     else if (waves1 >= 4096) gemv_kernel<B32, RESCALE, MR, 2><<<dim3((unsigned)((p.N + 1) / 2), (unsigned)G), dim3(256), 0, 0>>>(p);
     else gemv_kernel<B32, RESCALE, MR, 4><<<dim3((unsigned)p.N, (unsigned)G), dim3(256), 0, 0>>>(p);
+}
+
+bool gemm_gemv_grouped_launch(const GroupedDesc &d)
+{
+    if (d.rows < 1 || d.rows > 65535 || d.N < 1 || d.K < 1 || d.groups < 1) return false;
+    ValuParams p = {};
+    p.A = d.A; p.B = nullptr; p.C = d.C; p.R = d.R;
+    p.lda = d.lda; p.sA = d.lda; p.ldbn = d.K; p.ldbk = 1; p.sB = 0; p.ldc = d.ldc; p.sC = d.ldc;
+    p.M = 1; p.N = d.N; p.K = d.K; p.shift = d.shift;
+    p.init = d.init; p.a_rs = 1; p.b_rs = 1; p.a_shift = 0; p.b_shift = 0;
+    p.grp_b = d.B; p.grp_seg = d.seg; p.groups = d.groups;
+    // 16-byte loads: rows of A by their pointer and stride; every expert's B is taken to start on a 16-byte boundary
+    // (a tensor of its own), its rows follow from K
+    const size_t esz = d.b32 ? 4 : 8;
+    p.tiles_m = ((((uintptr_t)d.A | (uintptr_t)(d.lda * 8)) & 15) == 0 && ((size_t)d.K * esz) % 16 == 0) ? 1 : 0;
+    const long waves1 = (long)d.N * d.rows;
+    const unsigned rows = (unsigned)d.rows;
+#define ZK_GEMVG(B32) do {                                                                                                  \
+        if (waves1 >= 8192) gemv_kernel<B32, false, 1, 1, true><<<dim3((unsigned)((d.N + 3) / 4), rows), dim3(256), 0, 0>>>(p);      \
+        else if (waves1 >= 4096) gemv_kernel<B32, false, 1, 2, true><<<dim3((unsigned)((d.N + 1) / 2), rows), dim3(256), 0, 0>>>(p);  \
+        else gemv_kernel<B32, false, 1, 4, true><<<dim3((unsigned)d.N, rows), dim3(256), 0, 0>>>(p);                                  \
+    } while (0)
+    if (d.b32) ZK_GEMVG(true); else ZK_GEMVG(false);
+#undef ZK_GEMVG
+    return true;
 }
 
 bool gemm_gemv_launch(const GemmDesc &d)
