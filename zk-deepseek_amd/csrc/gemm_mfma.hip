@@ -966,7 +966,7 @@ static const Instance *instances(int *count)
         ZK_PROBE
 #else
         make_instance<3, 3>(), make_instance<4, 3>(), make_instance<4, 4>(), make_instance<5, 4>(),
-        make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(),
+        make_instance<5, 5>(), make_instance<6, 5>(), make_instance<3, 5>(), make_instance<6, 3>(), make_instance<4, 5>(),
         make_instance<9, 5>(), make_instance<5, 9>(), make_instance<9, 9>(),
         make_instance<3, 3, true>(), make_instance<5, 5, true>(),
         // 28-bit activations against 31-bit weights: what an expert sees after the norm (inference/model.py:1017, 1324)
