@@ -474,6 +474,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     const bool verify_a = !APL && tn < vmod_a;
     const bool verify_b = tm < vmod_b && (g == 0 || p.verify_b_all_batches);
     MinMax ra = { INT64_MAX, INT64_MIN }, rb = { INT64_MAX, INT64_MIN };
+    int rb32_lo = INT32_MAX, rb32_hi = INT32_MIN;        // the range of an int32 B is tracked in 32 bits and joins rb at the end
 
     v16i acc[WM][WN][D];
 #pragma unroll
@@ -680,7 +681,16 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 #pragma unroll
             for (int it = 0; it < B_IT; it++)
 #pragma unroll
-                for (int q = 0; q < 8; q++) mm_update(rb, BRS ? tdiv_pow2(sb[it][q], p.b_shift) : sb[it][q]);     // what the digits are taken from
+                for (int q = 0; q < 8; q++) {
+                    if (B32 && !BRS) {
+                        // int32 values: one min and one max instruction each, against four for a 64-bit pair
+                        const int v = (int)sb[it][q];
+                        rb32_lo = v < rb32_lo ? v : rb32_lo;
+                        rb32_hi = v > rb32_hi ? v : rb32_hi;
+                    } else {
+                        mm_update(rb, BRS ? tdiv_pow2(sb[it][q], p.b_shift) : sb[it][q]);     // what the digits are taken from
+                    }
+                }
         }
     };
 
@@ -734,6 +744,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     if (verify_a || verify_b) {
         __syncthreads();
         MinMax *red = reinterpret_cast<MinMax *>(smem);
+        if (B32 && !BRS && rb32_lo <= rb32_hi) mm_merge(rb, MinMax{ (int64_t)rb32_lo, (int64_t)rb32_hi });
         ra = mm_wave(ra);
         rb = mm_wave(rb);
         if (lane == 0) { red[2 * wave] = ra; red[2 * wave + 1] = rb; }
