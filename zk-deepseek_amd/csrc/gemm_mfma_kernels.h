@@ -670,14 +670,19 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     const int ks_begin = (int)((long)sidx * ksteps / nsplit), ks_end = (int)((long)(sidx + 1) * ksteps / nsplit);
 
     // Range tracking of the staged elements of data step d, done while the registers still hold them.
-    auto track = [&](int d) {
-        if (verify_a && d % vmod_a == tn) {
+    // (called once per data step, in order: the turn counters stand for d % vmod_a and d % vmod_b without a division)
+    int turn_a = ks_begin % vmod_a, turn_b = ks_begin % vmod_b;
+    auto track = [&](int) {
+        const bool my_a = turn_a == tn, my_b = turn_b == tm;
+        turn_a = turn_a + 1 == vmod_a ? 0 : turn_a + 1;
+        turn_b = turn_b + 1 == vmod_b ? 0 : turn_b + 1;
+        if (verify_a && my_a) {
 #pragma unroll
             for (int it = 0; it < A_IT; it++)
 #pragma unroll
                 for (int q = 0; q < 8; q++) mm_update(ra, sa[it][q]);
         }
-        if (verify_b && d % vmod_b == tm) {
+        if (verify_b && my_b) {
 #pragma unroll
             for (int it = 0; it < B_IT; it++)
 #pragma unroll
