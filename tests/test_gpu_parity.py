@@ -165,11 +165,11 @@ def test_gemm_head_projection_divisor_on_mfma(K, oracle, w32, b_rs):
     K.lib.zk_gemm_set_path(0)
 
 
-@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
 @pytest.mark.parametrize("w32", [False, True])
 def test_gemm_one_or_two_rows(K, oracle, M, w32):
-    """a decoding step: the matrix-vector kernel (automatic path) on narrow and wide outputs, odd K, unaligned rows,
-    batches, full-range operands, operand divisors and every shift class"""
+    """a decoding step: the matrix-vector kernel (automatic path; three or four rows in two passes) on narrow and wide
+    outputs, odd K, unaligned rows, batches, full-range operands, operand divisors and every shift class"""
     rng = np.random.default_rng(40 + M + w32)
     for Bd, Kd, N, bits_a, bits_w, c in ((1, 7168, 576, 20, 16, 29), (1, 1000, 5000, 37, 31, 30), (3, 333, 130, 63, 63, 0),
                                          (1, 1, 1, 63, 63, 63), (2, 4097, 9, 50, 40, 33), (1, 64, 20000, 31, 31, 16)):

@@ -181,6 +181,7 @@ void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard)
 // output.  Bytes in flight are what this kernel lives on: with 8-byte loads of int32 weights it streamed 1.7 TB/s,
 // with 16-byte loads 3.4 TB/s.
 constexpr int kGemvMaxM = 2;
+constexpr long kGemvTwoPassBytes = 64L << 20;
 
 // A 128-bit sum kept as a 64-bit low word and a count of what went past it, so that adding a signed 64-bit product is
 // four independent-looking instructions (sign word, add, add-with-carry twice) instead of a four-word carry chain.
@@ -417,6 +418,20 @@ bool gemm_gemv_grouped_launch(const GroupedDesc &d)
 
 bool gemm_gemv_launch(const GemmDesc &d)
 {
+    // three or four rows: two passes of two rows while the matrix is small enough for the launch count to matter more
+    // than a second pass over it (the MFMA route is four launches however small the product)
+    if (d.M > kGemvMaxM && d.M <= 2 * kGemvMaxM && d.G >= 1 && d.N >= 1 && d.K >= 1 &&
+        (long)d.G * d.N * d.K * (d.b32 ? 4 : 8) <= kGemvTwoPassBytes) {
+        for (int m0 = 0; m0 < d.M; m0 += kGemvMaxM) {
+            GemmDesc h = d;
+            h.M = d.M - m0 < kGemvMaxM ? d.M - m0 : kGemvMaxM;
+            h.A = d.A + (long)m0 * d.lda;
+            h.C = d.C + (long)m0 * d.ldc;
+            h.R = d.R ? d.R + (long)m0 * d.ldc : nullptr;
+            if (!gemm_gemv_launch(h)) return false;        // (the checks below do not depend on the row count)
+        }
+        return true;
+    }
     if (d.M < 1 || d.M > kGemvMaxM || d.G > 65535 || d.N < 1 || d.K < 1) return false;
     const bool kmajor = d.ldbn == 1 && d.ldbk != 1;
     if (!kmajor && d.ldbk != 1) return false;
