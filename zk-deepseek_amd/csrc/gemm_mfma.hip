@@ -18,8 +18,8 @@
 // fetched by exactly one load instruction.
 //
 // The digit counts are speculated from a cached or sampled range.  The kernels track the exact min and max of
-// everything they load (every workgroup leaves its share in a slot of its own, a one-workgroup kernel folds
-// them and compares with the digit counts used).  The first call for an operand reads the verdict back and
+// everything they load (every workgroup leaves its share in a slot of its own, a few workgroups fold
+// them and compare with the digit counts used).  The first call for an operand reads the verdict back and
 // reruns with wider digits if the guess was too small.  Later calls do not wait: a guarded launch of the
 // vector-ALU kernel follows, which recomputes everything if the verdict is bad and returns at once otherwise,
 // and the exact range travels to the host behind the stream to refresh the cache.  Results never depend on

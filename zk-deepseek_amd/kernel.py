@@ -295,16 +295,6 @@ def quantize_bf16(param: torch.Tensor, k: int, dtype=torch.int32) -> torch.Tenso
 atexit.register(lambda: lib.zk_dump_flush())
 
 
-def saveTensor(fileName, t):
-    """Raw C-order little-endian bytes, the witness format the proving side reads back."""
-    t = t.detach()
-    if t.device.type != "cpu":
-        t = t.cpu()
-    t = t.contiguous()
-    with open(fileName, "wb") as f:
-        f.write(t.numpy().tobytes(order="C"))
-
-
 LOG_TABLE_SIZE = 8
 EXP2_FRAC_LUT_Q21 = None
 EXP2_FRAC_LUT_Q19 = None
