@@ -206,6 +206,31 @@ def test_gemm_one_or_two_rows(K, oracle, M, w32):
     assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
 
 
+@pytest.mark.parametrize("M", [1, 2])
+def test_gemm_rows_staged_in_lds(K, oracle, M):
+    """one or two rows against int32 weights with K % 4 == 0 and a wide output: the kernel that stages the rows in LDS as
+    three 21-bit pieces (several staging rounds, one, two and four columns per wave with ragged last workgroups, strided
+    batches, shifts 0 and 63, and the operands that bring its 64-bit accumulators closest to their limit)"""
+    rng = np.random.default_rng(70 + M)
+    for Bd, Kd, N, bits_a, c in ((1, 9000, 2100, 63, 29), (1, 520, 16390, 40, 0), (1, 516, 9001, 63, 63), (3, 512, 900, 31, 17),
+                                 (1, 256, 3000, 63, 31)):
+        A = rand_i64(rng, (Bd, M, Kd), bits_a)
+        W = rand_i32(rng, (N, Kd), 31)
+        A[0, 0, :3] = [-(1 << 63), (1 << 63) - 1, -1]
+        W[0, :3] = [-(1 << 31), (1 << 31) - 1, -(1 << 31)]
+        _gemm_case(K, oracle, 0, A, W, 1, 1, c)
+        assert K.gemm_last_plan()[0] == 1
+    # the longest K it takes, every product at its largest magnitude and of one sign per column
+    Kd, N = 65536, 2048
+    A = np.full((1, M, Kd), -(1 << 63), np.int64)
+    A[0, M - 1, 1::2] = (1 << 63) - 1
+    W = np.full((N, Kd), -(1 << 31), np.int32)
+    W[1::2] = (1 << 31) - 1
+    W[2, ::3] = 12345
+    _gemm_case(K, oracle, 0, A, W, 1, 1, 33)
+    assert K.gemm_last_plan()[0] == 1
+
+
 def test_gemm_rejects_bad_arguments(K):
     A = torch.zeros((1, 2, 3), dtype=torch.int64, device="cuda")
     W = torch.zeros((4, 3), dtype=torch.int64, device="cuda")
@@ -859,10 +884,12 @@ def test_int64_grouped_bmm(K, oracle, path, w32, bits):
 
 
 @pytest.mark.parametrize("w32", [False, True])
-@pytest.mark.parametrize("T,Kr,Kd,N", [(1, 8, 520, 300), (2, 8, 7168, 64), (4, 3, 333, 1030), (1, 1, 64, 5000)])
+@pytest.mark.parametrize("T,Kr,Kd,N", [(1, 8, 520, 300), (2, 8, 7168, 64), (4, 3, 333, 1030), (1, 1, 64, 5000), (8, 8, 520, 300),
+                                       (1, 8, 8200, 300), (2, 8, 260, 4200)])
 def test_int64_grouped_bmm_few_rows(K, oracle, w32, T, Kr, Kd, N):
-    """a decoding step's routed experts: up to 32 rows go row by row through the matrix-vector kernel in one launch
-    (every row against the weights of its own expert, empty experts in between, odd K, the remainder output)"""
+    """a decoding step's routed experts: up to 32 rows (64 with int32 weights and K % 4 == 0) go row by row through the
+    matrix-vector kernels in one launch (every row against the weights of its own expert, empty experts in between, odd
+    K, several staging rounds, the remainder output)"""
     rng = np.random.default_rng(T * 100 + Kr + w32)
     E = 16
     idx = _routing(rng, T, E, Kr)
@@ -879,7 +906,8 @@ def test_int64_grouped_bmm_few_rows(K, oracle, w32, T, Kr, Kd, N):
         Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
         assert np.array_equal(host(C), Ce), "quotient"
         assert np.array_equal(host(R), Re), "remainder"
-    assert K.lib.zk_gemm_grouped_mfma_calls() == before and K.gemm_last_plan()[0] == 1
+    if T * Kr <= 32 or w32:
+        assert K.lib.zk_gemm_grouped_mfma_calls() == before and K.gemm_last_plan()[0] == 1
 
 
 @pytest.mark.parametrize("w32", [False, True])

@@ -34,9 +34,11 @@ void gemm_dispatch(const char *name, const GemmDesc &d)
     check_launch(name);
 }
 
-// rows up to which the grouped product runs row by row on the matrix-vector kernel (one or two tokens at top-8):
-// measured, 8 rows take 0.45 ms there against 0.95 ms on the 32-row MFMA kernels, 64 rows take as long on either
-constexpr int kGroupedGemvMaxRows = 32;
+// rows up to which the grouped product is offered to the matrix-vector kernels, which go row by row (a few tokens at
+// top-8).  Measured on config 5's experts with int32 weights: 8 rows 0.27 ms against 0.95 ms on the 32-row MFMA kernels,
+// 64 rows 1.85 against 2.18 ms, 128 rows 3.4 against 3.3 ms.  (The launcher itself stops at 32 rows for products that
+// its LDS-staged kernel does not take.)
+constexpr int kGroupedGemvMaxRows = 64;
 
 void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
 {

@@ -32,6 +32,7 @@ struct ValuParams {
     const void *const *grp_b;                 // device array of `groups` device pointers
     const int *grp_seg;                       // device [groups + 1]: first row of every segment
     int groups;
+    int chunk;                                // staged matrix-vector kernel: elements of A per staging round
 };
 
 template <bool B32>
@@ -346,6 +347,169 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
     }
 }
 
+// One row of A against int32 weights with the row staged in LDS.  Every wave of a workgroup needs the whole row, and
+// read from memory it costs twice the bytes of the weights it meets; staged once per workgroup it is split on the way in,
+//     a = a2 * 2^42 + a1 * 2^21 + a0,   a0, a1 in [0, 2^21),   a2 in [-2^21, 2^21),
+// so that a piece times an int32 weight stays below 2^52 in magnitude and a lane can add 1024 of them in a plain 64-bit
+// accumulator: one v_mad_i64_i32 per piece, no carry bookkeeping, and the vector memory pipe carries weights only.
+// The three sums of a column meet in 128 bits at the end.  K <= 65536 (1024 terms per lane), K % 4 == 0, 16-byte
+// aligned rows of A and B (decided on the host).  A wave owns CPW consecutive columns.
+#ifndef ZK_STAGED_WAVES
+#define ZK_STAGED_WAVES 8
+#endif
+#ifndef ZK_STAGED_UN
+#define ZK_STAGED_UN 8
+#endif
+#ifndef ZK_STAGED_CHUNK
+#define ZK_STAGED_CHUNK 4096
+#endif
+constexpr int kStagedWaves = ZK_STAGED_WAVES;
+constexpr int kStagedChunk = ZK_STAGED_CHUNK;     // elements of A per staging round: 12 bytes of LDS each
+constexpr int kStagedMaxK = 65536;
+
+typedef int v4i_s __attribute__((ext_vector_type(4)));
+
+template <int MR, int CPW, bool GRP>
+__global__ __launch_bounds__(64 * kStagedWaves) void gemv32_staged_kernel(ValuParams p)
+{
+    constexpr int UN = ZK_STAGED_UN / MR, T = 64 * kStagedWaves;      // 16-byte loads of weights in flight per lane
+    extern __shared__ __align__(16) int32_t staged[];          // [MR][3] planes of `chunk` elements
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = blockIdx.y;
+    const int64_t *Ag = p.A + (long)g * p.sA;
+    const int32_t *Bbase = reinterpret_cast<const int32_t *>(p.B) + (long)g * p.sB;
+    if (GRP) {
+        // the segment that holds row g: the last one that starts at or before it
+        int lo = 0, hi = p.groups - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (p.grp_seg[mid] <= g) lo = mid; else hi = mid - 1;
+        }
+        Bbase = reinterpret_cast<const int32_t *>(p.grp_b[lo]);
+    }
+    const int chunk = p.chunk;
+    const v4i_s *plane[MR][3];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int i = 0; i < 3; i++) plane[m][i] = reinterpret_cast<const v4i_s *>(staged + (3 * m + i) * chunk);
+    const long n_first = ((long)blockIdx.x * kStagedWaves + wave) * CPW;
+    int64_t acc[MR][CPW][3];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int c = 0; c < CPW; c++) acc[m][c][0] = acc[m][c][1] = acc[m][c][2] = 0;
+
+    for (int k0 = 0; k0 < p.K; k0 += chunk) {
+        const int len = p.K - k0 < chunk ? p.K - k0 : chunk;
+        if (k0) __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            int2 *s0 = reinterpret_cast<int2 *>(staged + (3 * m) * chunk), *s1 = reinterpret_cast<int2 *>(staged + (3 * m + 1) * chunk),
+                 *s2 = reinterpret_cast<int2 *>(staged + (3 * m + 2) * chunk);
+            for (int k = 2 * threadIdx.x; k < len; k += 2 * T) {
+                const longlong2 t = *reinterpret_cast<const longlong2 *>(Ag + (long)m * p.lda + k0 + k);
+                s0[k >> 1] = make_int2((int)((uint32_t)t.x & 0x1FFFFFu), (int)((uint32_t)t.y & 0x1FFFFFu));
+                s1[k >> 1] = make_int2((int)((uint32_t)(t.x >> 21) & 0x1FFFFFu), (int)((uint32_t)(t.y >> 21) & 0x1FFFFFu));
+                s2[k >> 1] = make_int2((int)(t.x >> 42), (int)(t.y >> 42));
+            }
+        }
+        __syncthreads();
+        const int units = len >> 2;
+#pragma unroll
+        for (int c = 0; c < CPW; c++) {
+            const long n = n_first + c < p.N ? n_first + c : p.N - 1;      // columns past N read the last row; dropped below
+            const v4i_s *brow = reinterpret_cast<const v4i_s *>(Bbase + n * p.ldbn + k0);
+            for (int q0 = 0; q0 < units; q0 += 64 * UN) {
+                v4i_s b[UN];
+#pragma unroll
+                for (int u = 0; u < UN; u++) {
+                    const int q = q0 + u * 64 + lane;
+                    b[u] = q < units ? __builtin_nontemporal_load(brow + q) : v4i_s{ 0, 0, 0, 0 };
+                }
+#pragma unroll
+                for (int u = 0; u < UN; u++) {
+                    int q = q0 + u * 64 + lane;
+                    q = q < units ? q : units - 1;                           // (its weights are zero)
+#pragma unroll
+                    for (int m = 0; m < MR; m++)
+#pragma unroll
+                        for (int i = 0; i < 3; i++) {
+                            const v4i_s x = plane[m][i][q];
+                            acc[m][c][i] += (int64_t)x.x * b[u].x + (int64_t)x.y * b[u].y + (int64_t)x.z * b[u].z + (int64_t)x.w * b[u].w;
+                        }
+                }
+            }
+        }
+    }
+
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int c = 0; c < CPW; c++) {
+            u128 sum = (u128)((i128)acc[m][c][0] + ((i128)acc[m][c][1] << 21) + ((i128)acc[m][c][2] << 42));
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const uint64_t lo = (uint64_t)__shfl_xor((long long)(uint64_t)sum, off, 64);
+                const uint64_t hi = (uint64_t)__shfl_xor((long long)(uint64_t)(sum >> 64), off, 64);
+                sum += ((u128)hi << 64) | lo;
+            }
+            if (lane == 0 && n_first + c < p.N) {
+                sum += (u128)(i128)p.init;
+                const long o = (long)g * p.sC + (long)m * p.ldc + n_first + c;
+                p.C[o] = (int64_t)(uint64_t)((i128)sum >> p.shift);
+                if (p.R) p.R[o] = (int64_t)((uint64_t)sum & rmask);
+            }
+        }
+}
+
+static int device_cus()
+{
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
+// Launches the staged kernel if the product is one it takes: one or two rows (per batch or segment row), int32 weights,
+// no divisors, K a multiple of four up to kStagedMaxK, 16-byte aligned rows, and enough columns for a workgroup per
+// compute unit (a narrower output is better served by waves that share a column along K).
+template <bool GRP>
+static bool gemv32_staged_launch(ValuParams p, long rows, int cus)
+{
+    if (p.K % 4 != 0 || p.K > kStagedMaxK || p.K < 256 || rows > 65535 || p.M < 1 || p.M > 2) return false;
+    const long wg1 = ((p.N + kStagedWaves - 1) / kStagedWaves) * rows;
+    if (wg1 < cus) return false;
+    p.chunk = p.K < kStagedChunk / p.M ? p.K : kStagedChunk / p.M;      // 48 KB of LDS: three workgroups per compute unit
+    const size_t lds = (size_t)3 * p.M * p.chunk * sizeof(int32_t);
+    // more columns per wave (the staging is shared by more of them) while that leaves two workgroups per compute unit
+    const long wg4 = ((p.N + 4 * kStagedWaves - 1) / (4 * kStagedWaves)) * rows;
+    const long wg2 = ((p.N + 2 * kStagedWaves - 1) / (2 * kStagedWaves)) * rows;
+    auto launch = [&](auto mr_tag, auto cpw_tag) {
+        constexpr int MR = decltype(mr_tag)::value, CPW = decltype(cpw_tag)::value;
+        auto fn = gemv32_staged_kernel<MR, CPW, GRP>;
+        static bool raised = false;
+        if (lds > 64 * 1024 && !raised) {
+            if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { (void)hipGetLastError(); return false; }
+            raised = true;
+        }
+        const dim3 grid((unsigned)((p.N + CPW * kStagedWaves - 1) / (CPW * kStagedWaves)), (unsigned)rows);
+        fn<<<grid, dim3(64 * kStagedWaves), lds, 0>>>(p);
+        return true;
+    };
+    typedef std::integral_constant<int, 1> I1;
+    typedef std::integral_constant<int, 2> I2;
+    typedef std::integral_constant<int, 4> I4;
+    if (p.M == 2) return wg2 >= 2L * cus ? launch(I2(), I2()) : launch(I2(), I1());
+    if (wg4 >= 2L * cus) return launch(I1(), I4());
+    if (wg2 >= 2L * cus) return launch(I1(), I2());
+    return launch(I1(), I1());
+}
+
 // The same for n-contiguous B (the per-head weights of `bshd,hdc->bshc`): a lane owns an output column and walks K, the
 // loads of a row of B are contiguous over the wave, and the elements of A are the same for every lane.
 template <bool B32, bool RESCALE, int MR>
@@ -404,6 +568,8 @@ bool gemm_gemv_grouped_launch(const GroupedDesc &d)
     // (a tensor of its own), its rows follow from K
     const size_t esz = d.b32 ? 4 : 8;
     p.tiles_m = ((((uintptr_t)d.A | (uintptr_t)(d.lda * 8)) & 15) == 0 && ((size_t)d.K * esz) % 16 == 0) ? 1 : 0;
+    if (d.b32 && p.tiles_m && gemv32_staged_launch<true>(p, d.rows, device_cus())) return true;
+    if (d.rows > 32) return false;         // past that the 32-row MFMA kernels are as fast as the kernel below
     const long waves1 = (long)d.N * d.rows;
     const unsigned rows = (unsigned)d.rows;
 #define ZK_GEMVG(B32) do {                                                                                                  \
@@ -465,6 +631,7 @@ bool gemm_gemv_launch(const GemmDesc &d)
 #undef ZK_GEMVK
         return true;
     }
+    if (d.b32 && !rescale && p.tiles_m && gemv32_staged_launch<false>(p, d.G, device_cus())) return true;
 #define ZK_GEMV(B32, RS) do { if (d.M == 1) gemv_launch3<B32, RS, 1>(p, d.G); else gemv_launch3<B32, RS, 2>(p, d.G); } while (0)
     if (d.b32) { if (rescale) ZK_GEMV(true, true); else ZK_GEMV(true, false); }
     else { if (rescale) ZK_GEMV(false, true); else ZK_GEMV(false, false); }
