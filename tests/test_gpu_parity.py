@@ -837,7 +837,7 @@ def _routing(rng, T, E, Kr):
     return np.stack([rng.permutation(live)[:Kr] for _ in range(T)]).astype(np.int64)
 
 
-@pytest.mark.parametrize("T,E,Kr", [(1, 8, 2), (5, 4, 4), (100, 16, 3), (256, 256, 8), (700, 32, 6)])
+@pytest.mark.parametrize("T,E,Kr", [(1, 8, 2), (5, 4, 4), (100, 16, 3), (256, 256, 8), (700, 32, 6), (300, 700, 4), (2000, 257, 1)])
 def test_moe_dispatch(K, oracle, T, E, Kr):
     rng = np.random.default_rng(T + E)
     idx = _routing(rng, T, E, Kr)

@@ -67,13 +67,16 @@ __global__ __launch_bounds__(256) void gate_route_kernel(const int64_t *__restri
     if (n_groups > 1) {
         // lane g ends up holding the score of group g
         const int gsize = E / n_groups;
+        int grp[EPL];                                     // group of every element (one division each, not one per test)
+#pragma unroll
+        for (int j = 0; j < EPL; j++) grp[j] = live[j] ? (lane * EPL + j) / gsize : -1;
         int64_t my_group_score = 0;
         for (int g = 0; g < n_groups; g++) {
             Best b1 = { INT64_MIN, kNone };
 #pragma unroll
             for (int j = 0; j < EPL; j++) {
                 const int e = lane * EPL + j;
-                if (live[j] && e / gsize == g) b1 = better(b1, Best{ s[j], e });
+                if (grp[j] == g) b1 = better(b1, Best{ s[j], e });
             }
             b1 = wave_best(b1);
             int64_t gs = b1.v;
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(const int64_t *__restri
 #pragma unroll
                 for (int j = 0; j < EPL; j++) {
                     const int e = lane * EPL + j;
-                    if (live[j] && e / gsize == g && e != b1.idx) b2 = better(b2, Best{ s[j], e });
+                    if (grp[j] == g && e != b1.idx) b2 = better(b2, Best{ s[j], e });
                 }
                 b2 = wave_best(b2);
                 gs = (int64_t)((uint64_t)gs + (uint64_t)(b2.idx == kNone ? 0 : b2.v));
@@ -98,8 +101,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(const int64_t *__restri
         const int keep = (lane < n_groups && rank < topk_groups) ? 1 : 0;
 #pragma unroll
         for (int j = 0; j < EPL; j++) {
-            const int e = lane * EPL + j;
-            const int kept = __shfl(keep, live[j] ? e / gsize : 0, kWave);
+            const int kept = __shfl(keep, live[j] ? grp[j] : 0, kWave);
             if (live[j] && !kept) s[j] = kMasked;
         }
     }

@@ -27,23 +27,39 @@ __global__ __launch_bounds__(256) void moe_count_kernel(const int64_t *__restric
     if (threadIdx.x == 0) counts[e] = red[0] + red[1] + red[2] + red[3];
 }
 
-// exclusive scan of the counts and the table of 32-row tiles; one thread (E is at most a few hundred)
-__global__ void moe_scan_kernel(const int *__restrict__ counts, int E, int *__restrict__ seg, int *__restrict__ tiles,
-                                int *__restrict__ ntiles)
+// exclusive scan of the counts and the table of 32-row tiles: one workgroup, 256 experts per round (a single thread
+// walking 256 counts took 19 us, longer than every other step of a one-token dispatch)
+__global__ __launch_bounds__(256) void moe_scan_kernel(const int *__restrict__ counts, int E, int *__restrict__ seg, int *__restrict__ tiles,
+                                                       int *__restrict__ ntiles)
 {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int row = 0, nt = 0;
-    for (int e = 0; e < E; e++) {
-        seg[e] = row;
-        for (int r = 0; r < counts[e]; r += 32) {
-            tiles[2 * nt] = e;
-            tiles[2 * nt + 1] = row + r;
-            nt++;
+    __shared__ int wave_sum[2][4];
+    __shared__ int carry[2];                       // rows and tiles of the rounds before this one
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) carry[0] = carry[1] = 0;
+    __syncthreads();
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int e = e0 + (int)threadIdx.x;
+        const int c = e < E ? counts[e] : 0, t = (c + 31) >> 5;
+        int pc = c, pt = t;                        // inclusive prefix sums over the wave
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int vc = __shfl_up(pc, off, 64), vt = __shfl_up(pt, off, 64);
+            if (lane >= off) { pc += vc; pt += vt; }
         }
-        row += counts[e];
+        if (lane == 63) { wave_sum[0][wave] = pc; wave_sum[1][wave] = pt; }
+        __syncthreads();
+        int bc = carry[0], bt = carry[1];
+        for (int w = 0; w < wave; w++) { bc += wave_sum[0][w]; bt += wave_sum[1][w]; }
+        if (e < E) {
+            const int row = bc + pc - c, tile = bt + pt - t;
+            seg[e] = row;
+            for (int i = 0; i < t; i++) { tiles[2 * (tile + i)] = e; tiles[2 * (tile + i) + 1] = row + 32 * i; }
+        }
+        __syncthreads();
+        if (threadIdx.x == 255) { carry[0] = bc + pc; carry[1] = bt + pt; }
+        __syncthreads();
     }
-    seg[E] = row;
-    ntiles[0] = nt;
+    if (threadIdx.x == 0) { seg[E] = carry[0]; ntiles[0] = carry[1]; }
 }
 
 // workgroup e walks the entries in order and gives its own consecutive rows: a stable partition
@@ -125,7 +141,7 @@ void moe_dispatch(const int64_t *indices, int T, int K, int E, int *counts_scrat
     if (E > 65535) { zk::set_error(zk::kUnsupportedSize, "%s: more than 65535 experts", name); return; }
     const long entries = (long)T * K;
     zk::moe_count_kernel<<<dim3((unsigned)E), dim3(256), 0, 0>>>(indices, entries, counts_scratch);
-    zk::moe_scan_kernel<<<dim3(1), dim3(64), 0, 0>>>(counts_scratch, E, seg, tiles, ntiles);
+    zk::moe_scan_kernel<<<dim3(1), dim3(256), 0, 0>>>(counts_scratch, E, seg, tiles, ntiles);
     if (entries > 0) zk::moe_place_kernel<<<dim3((unsigned)E), dim3(256), 0, 0>>>(indices, entries, K, seg, sorted_token, sorted_pos);
     zk::check_launch(name);
 }
