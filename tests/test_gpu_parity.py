@@ -380,6 +380,22 @@ def test_einsums_model_shapes(K, oracle, path):
 
 
 # ---------------------------------------------------------------------------------- softmax -----
+def test_einsum_values_rewritten_with_contiguous_rows(K, oracle, monkeypatch):
+    """`bsht,btc->bshc` on the MFMA path copies a small n-contiguous int64 B into row-major scratch first (products of
+    2^32 MACs and more; the threshold is lowered here): ragged T and C, two batches, and a second call with another B
+    through the same scratch"""
+    monkeypatch.setenv("ZK_B_ROWS_MIN_MACS", "1")
+    rng = np.random.default_rng(77)
+    K.lib.zk_gemm_set_path(2)
+    for Bq, S, H, T, Cc in ((2, 9, 5, 70, 45), (1, 40, 3, 33, 130), (1, 3, 16, 257, 64)):
+        for rep in range(2):
+            pr = rng.integers(0, 1 << 19, size=(Bq, S, H, T), dtype=np.int64)
+            kv = rand_i64(rng, (Bq, T, Cc), 36 if rep else 24)
+            assert np.array_equal(host(K.einsum_bsht_btc_bshc(dev(pr), dev(kv), 23)), oracle.einsum_bsht_btc_bshc(pr, kv, 23)), (Bq, S, H, T, Cc, rep)
+            assert K.gemm_last_plan()[0] == 2
+    K.lib.zk_gemm_set_path(0)
+
+
 def _scores(rng, shape, Q, masked=True):
     x = rng.integers(-(12 << Q), 12 << Q, size=shape, dtype=np.int64)
     if masked and shape[-1] > 1:
