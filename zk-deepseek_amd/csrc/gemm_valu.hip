@@ -354,17 +354,9 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
 // accumulator: one v_mad_i64_i32 per piece, no carry bookkeeping, and the vector memory pipe carries weights only.
 // The three sums of a column meet in 128 bits at the end.  K <= 65536 (1024 terms per lane), K % 4 == 0, 16-byte
 // aligned rows of A and B (decided on the host).  A wave owns CPW consecutive columns.
-#ifndef ZK_STAGED_WAVES
-#define ZK_STAGED_WAVES 8
-#endif
-#ifndef ZK_STAGED_UN
-#define ZK_STAGED_UN 8
-#endif
-#ifndef ZK_STAGED_CHUNK
-#define ZK_STAGED_CHUNK 4096
-#endif
-constexpr int kStagedWaves = ZK_STAGED_WAVES;
-constexpr int kStagedChunk = ZK_STAGED_CHUNK;     // elements of A per staging round: 12 bytes of LDS each
+constexpr int kStagedWaves = 8;
+constexpr int kStagedLoads = 8;          // 16-byte loads of weights in flight per lane (shared out over the rows)
+constexpr int kStagedChunk = 4096;       // elements of A per staging round (over all rows): 12 bytes of LDS each
 constexpr int kStagedMaxK = 65536;
 
 typedef int v4i_s __attribute__((ext_vector_type(4)));
@@ -372,7 +364,7 @@ typedef int v4i_s __attribute__((ext_vector_type(4)));
 template <int MR, int CPW, bool GRP>
 __global__ __launch_bounds__(64 * kStagedWaves) void gemv32_staged_kernel(ValuParams p)
 {
-    constexpr int UN = ZK_STAGED_UN / MR, T = 64 * kStagedWaves;      // 16-byte loads of weights in flight per lane
+    constexpr int UN = kStagedLoads / MR, T = 64 * kStagedWaves;
     extern __shared__ __align__(16) int32_t staged[];          // [MR][3] planes of `chunk` elements
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = blockIdx.y;
@@ -491,12 +483,8 @@ static bool gemv32_staged_launch(ValuParams p, long rows, int cus)
     const long wg2 = ((p.N + 2 * kStagedWaves - 1) / (2 * kStagedWaves)) * rows;
     auto launch = [&](auto mr_tag, auto cpw_tag) {
         constexpr int MR = decltype(mr_tag)::value, CPW = decltype(cpw_tag)::value;
+        static_assert(3 * kStagedChunk * sizeof(int32_t) <= 64 * 1024, "the staging planes fit the default dynamic LDS limit");
         auto fn = gemv32_staged_kernel<MR, CPW, GRP>;
-        static bool raised = false;
-        if (lds > 64 * 1024 && !raised) {
-            if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { (void)hipGetLastError(); return false; }
-            raised = true;
-        }
         const dim3 grid((unsigned)((p.N + CPW * kStagedWaves - 1) / (CPW * kStagedWaves)), (unsigned)rows);
         fn<<<grid, dim3(64 * kStagedWaves), lds, 0>>>(p);
         return true;
