@@ -182,6 +182,15 @@ def main():
         Wm = randint(g4, -(1 << 31), 1 << 31, (N, Kd)).to(torch.int32).cuda()
         extra["gemm_config4_q31_x_int32"] = gemm_leg(K, Am, Wm, 30, max(3, args.steps // 2), 1)
         del Am, Wm
+        # the headline shape with the weights prepared once as digit planes (zk_gemm_prepare_weights): what a model
+        # with static weights gets; the one-time preparation is timed separately and is NOT part of `value`
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        K.prepare_weights(W[0] if W.dim() == 3 else W)
+        prep_ms = (time.perf_counter() - t0) * 1e3
+        extra["gemm_config4_prepared_weights"] = gemm_leg(K, A, W, c, args.steps, 5)
+        extra["gemm_config4_prepared_weights"]["prepare_once_ms"] = prep_ms
+        K.release_weights(W[0] if W.dim() == 3 else W)
         # other instruction path on the headline shape, for the comparison
         K.lib.zk_gemm_set_path(1 if path == 2 else 2)
         extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1)
@@ -313,6 +322,18 @@ def main():
             hbm("moe_experts_config5_256tok_top8_of_256", lambda: K.moe_experts(xm, wm, im, tabs[0], tabs[1], tabs[2], False, 2048, 17, 20),
                 1, bytes_per_elem=wbytes, steps=3)
             extra["moe_experts_config5_256tok_top8_of_256"]["weight_bytes"] = wbytes
+            # the same with the experts' weights prepared once as digit planes (3 bytes per weight instead of 8)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for tb in tabs:
+                K.prepare_weights(tb, groups=256, N=int(2048 if tb is not tabs[2] else 7168), K=int(7168 if tb is not tabs[2] else 2048))
+            prep_ms = (time.perf_counter() - t0) * 1e3
+            hbm("moe_experts_config5_prepared_weights", lambda: K.moe_experts(xm, wm, im, tabs[0], tabs[1], tabs[2], False, 2048, 17, 20),
+                1, bytes_per_elem=wbytes * 3.0 / 8.0, steps=3)
+            extra["moe_experts_config5_prepared_weights"]["plane_bytes"] = wbytes * 3.0 / 8.0
+            extra["moe_experts_config5_prepared_weights"]["prepare_once_ms"] = prep_ms
+            for tb in tabs:
+                K.release_weights(tb)
             del ew1, ew3, ew2, tabs
             torch.cuda.empty_cache()
             # the same with the model's weight type: int32 at 31 bits (45 GB), shifts that keep the activations in Q23

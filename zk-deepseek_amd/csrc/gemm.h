@@ -41,7 +41,12 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 // Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
 // vector-ALU recomputation (known once their range has reached the host).
 long gemm_mfma_guard_hits();
-int gemm_mfma_last_pairs();       // digit pairs multiplied per element of K by the last MFMA launch
+// weights prepared once as digit planes (int64 matrices, or a device table of `groups` of them): 0 on success
+int gemm_mfma_prepare(const void *B, int groups, int N, int K);
+void gemm_mfma_release(const void *B);
+bool gemm_mfma_is_prepared(const void *B);
+int gemm_mfma_last_pairs();
+int gemm_mfma_last_prepared();    // 1 when the last MFMA launch read B from prepared planes       // digit pairs multiplied per element of K by the last MFMA launch
 
 // Grouped product: the rows of A and C form one contiguous segment per group and every group has its own
 // k-contiguous B[N,K] (the experts of a MoE layer after the tokens have been sorted by expert):

@@ -47,6 +47,7 @@ static const Instance *instances(int *count)
         mfma_instances_wide(t);
         mfma_instances_pruned(t);
         mfma_instances_rows32(t);
+        mfma_instances_rows32b(t);
 #endif
         return t;
     }();
@@ -55,7 +56,8 @@ static const Instance *instances(int *count)
 }
 
 // need_diag: the result's top bit is below 2^(8 need_diag), so diagonals from need_diag up cannot reach it
-static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int need_diag = 16)
+// exact_nb / variant: for B from prepared planes the instance must have exactly the planes' digit count and that kernel
+static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int need_diag = 16, int exact_nb = 0, int variant = -1)
 {
     int count;
     const Instance *t = instances(&count);
@@ -64,6 +66,8 @@ static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int 
     for (int i = 0; i < count; i++) {
         if (t[i].na < na || t[i].nb < nb || t[i].skinny != skinny) continue;
         if (t[i].dmax < 16 && t[i].dmax < need_diag) continue;
+        if (exact_nb && t[i].nb != exact_nb) continue;
+        if (variant >= 0 && !t[i].fn[variant]) continue;
         if (b32 && !t[i].fn[kB32Fly]) continue;
         if (!b32 && !t[i].fn[kB64Fly]) continue;
         long cost = kept_pairs_before(t[i].na, t[i].nb, t[i].dmax, t[i].na, 0);     // MFMAs per 32x32x32 block
@@ -156,16 +160,19 @@ static void drain_pending()
         const hipError_t st = hipEventQuery(s.ev);
         if (st != hipSuccess) { (void)hipGetLastError(); if (st == hipErrorNotReady) continue; }
         if (st == hipSuccess) {
-            g_cache.store_pair(s.key_a, limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip)),
-                               s.key_b, limbs_needed((int64_t)(s.host[2] ^ kSignFlip), (int64_t)(s.host[3] ^ kSignFlip)));
+            const int64_t b_lo = (int64_t)(s.host[2] ^ kSignFlip), b_hi = (int64_t)(s.host[3] ^ kSignFlip);
+            const int na_seen = limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip));
+            if (b_lo <= b_hi) g_cache.store_pair(s.key_a, na_seen, s.key_b, limbs_needed(b_lo, b_hi));
+            else g_cache.store(s.key_a, na_seen);            // B came from prepared planes: nothing of it was tracked
             if (s.host[4]) g_cache.guard_hits++;
         }
         s.busy = false;
     }
 }
 
-static int g_last_pairs = 0;
+static int g_last_pairs = 0, g_last_prepared = 0;
 int gemm_mfma_last_pairs() { return g_last_pairs; }
+int gemm_mfma_last_prepared() { return g_last_prepared; }
 
 long gemm_mfma_guard_hits()
 {
@@ -206,6 +213,126 @@ static FoldArgs make_fold(const unsigned long long *mm, long mm_count, const uns
     long parts = (mm_count + wg_count + kFoldSlotsPerPart - 1) / kFoldSlotsPerPart;
     parts = parts < 1 ? 1 : (parts > kFoldParts ? kFoldParts : parts);
     return FoldArgs{ mm, mm_count, wg, wg_count, range, na, nb, host_copy, (int)parts, g_cache.dev + 8 };
+}
+
+// ---- weights prepared once ------------------------------------------------------------------------------
+// Model weights do not change between calls.  `gemm_mfma_prepare` splits an int64 weight matrix (or every matrix of a
+// device table of pointers, the experts of a layer) into digit planes in MFMA fragment order once, with the digit
+// count its exact range needs; later launches whose B is that pointer copy the planes into LDS instead of splitting B
+// in every tile (and read NB bytes per weight instead of 8).  The original matrix stays the caller's and is what the
+// guarded vector-ALU fallback reads; the caller must not change it while it is prepared.
+struct PreparedB {
+    unsigned char *planes = nullptr;     // per matrix: [nsub][ksteps][nb] blocks of 1 KB
+    const void **table = nullptr;        // device array: the planes of every group (tables only)
+    int groups = 0, N = 0, K = 0, nb = 0, nsub = 0, ksteps = 0;
+};
+static std::map<const void *, PreparedB> g_prepared;
+
+static __global__ __launch_bounds__(256) void range_exact_kernel(const int64_t *__restrict__ x, long n, unsigned long long *out)
+{
+    MinMax r = { INT64_MAX, INT64_MIN };
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) mm_update(r, x[i]);
+    r = mm_wave(r);
+    if ((threadIdx.x & 63) == 0 && r.lo <= r.hi) {
+        atomicMin(out, (unsigned long long)r.lo ^ kSignFlip);
+        atomicMax(out + 1, (unsigned long long)r.hi ^ kSignFlip);
+    }
+}
+
+static void release_prepared(PreparedB &pb)
+{
+    if (pb.planes) (void)hipFree(pb.planes);
+    if (pb.table) (void)hipFree((void *)pb.table);
+    pb = PreparedB();
+}
+
+bool gemm_mfma_is_prepared(const void *B)
+{
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    return g_prepared.count(B) != 0;
+}
+
+void gemm_mfma_release(const void *B)
+{
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    auto it = g_prepared.find(B);
+    if (it == g_prepared.end()) return;
+    (void)hipDeviceSynchronize();              // launches that read the planes may still be under way
+    release_prepared(it->second);
+    g_prepared.erase(it);
+}
+
+int gemm_mfma_prepare(const void *B, int groups, int N, int K)
+{
+    const char *name = "zk_gemm_prepare_weights";
+    if (!B || groups < 0 || groups > 65535 || N < 1 || K < 1) { set_error(kBadArgument, "%s: bad argument", name); return 1; }
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    if (!init_cache()) return 1;
+    {
+        auto it = g_prepared.find(B);
+        if (it != g_prepared.end()) { (void)hipDeviceSynchronize(); release_prepared(it->second); g_prepared.erase(it); }
+    }
+    const int count = groups > 0 ? groups : 1;
+    std::vector<const void *> mats((size_t)count, B);
+    if (groups > 0 && hipMemcpy(mats.data(), B, (size_t)count * sizeof(void *), hipMemcpyDeviceToHost) != hipSuccess) {
+        set_error(kLaunchFailure, "%s: cannot read the pointer table", name);
+        return 1;
+    }
+    for (int i = 0; i < count; i++)
+        if (!mats[i]) { set_error(kBadArgument, "%s: null matrix in the table", name); return 1; }
+    // the exact range of all the matrices fixes one digit count for them
+    const long elems = (long)N * K;
+    range_reset_kernel<<<1, 64, 0, 0>>>(g_cache.dev);
+    const unsigned rgrid = (unsigned)(elems / 256 + 1 < 2048 ? elems / 256 + 1 : 2048);
+    for (int i = 0; i < count; i++)
+        range_exact_kernel<<<rgrid, 256, 0, 0>>>(reinterpret_cast<const int64_t *>(mats[i]), elems, g_cache.dev);
+    int64_t r[4];
+    if (!read_range(g_cache.dev, r)) { set_error(kLaunchFailure, "%s: range readback failed", name); return 1; }
+    const int need = limbs_needed(r[0], r[1]);
+    PreparedB pb;
+    pb.groups = groups; pb.N = N; pb.K = K;
+    pb.nb = need <= 3 ? 3 : (need <= 5 ? need : 9);              // digit counts the kernels are built for
+    pb.nsub = (N + 31) / 32;
+    pb.ksteps = (K + 31) / 32;
+    const size_t per = (size_t)pb.nsub * pb.ksteps * pb.nb * 1024;
+    if (hipMalloc(&pb.planes, per * count) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error(kLaunchFailure, "%s: cannot allocate %zu bytes of digit planes", name, per * count);
+        return 1;
+    }
+    if (groups > 0) {
+        std::vector<const void *> bases((size_t)count);
+        for (int i = 0; i < count; i++) bases[i] = pb.planes + per * i;
+        if (hipMalloc((void **)&pb.table, (size_t)count * sizeof(void *)) != hipSuccess ||
+            hipMemcpy((void *)pb.table, bases.data(), (size_t)count * sizeof(void *), hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            release_prepared(pb);
+            set_error(kLaunchFailure, "%s: cannot allocate the table of planes", name);
+            return 1;
+        }
+    }
+    // the pre-pass that splits A in fragment order does the same for the rows of a weight matrix (64 rows per workgroup)
+    const dim3 grid((unsigned)pb.ksteps, (unsigned)((pb.nsub * 32 + 63) / 64), 1);
+    if (!grow(g_cache.mm, g_cache.mm_count, (size_t)grid.x * grid.y * 2, "range scratch")) { release_prepared(pb); return 1; }
+    MfmaParams q = {};
+    q.lda = K; q.sA = 0; q.M = N; q.K = K;
+    for (int i = 0; i < count; i++) {
+        q.A = reinterpret_cast<const int64_t *>(mats[i]);
+        unsigned char *dst = pb.planes + per * i;
+        switch (pb.nb) {
+        case 3: a_planes_kernel<3, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
+        case 4: a_planes_kernel<4, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
+        case 5: a_planes_kernel<5, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
+        default: a_planes_kernel<9, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
+        }
+    }
+    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+        release_prepared(pb);
+        set_error(kLaunchFailure, "%s: the plane pre-pass failed", name);
+        return 1;
+    }
+    g_prepared[B] = pb;
+    return 0;
 }
 
 // B[g][k][n] (n contiguous) -> out[g][n][k]: 32x32 tiles through LDS, both sides coalesced
@@ -255,6 +382,14 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     MfmaParams p = {};
     p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
     p.lda = d.lda; p.sA = d.sA; p.ldbn = d.ldbn; p.ldbk = d.ldbk; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
+    // B prepared beforehand: its planes stand in for it, its digit count is exact
+    const PreparedB *prep = nullptr;
+    {
+        auto it = g_prepared.find(d.B);
+        if (it != g_prepared.end() && it->second.groups == 0 && !d.b32 && !kmajor && b_shift == 0 && d.sB == 0 && d.ldbk == 1 &&
+            d.ldbn == d.K && it->second.N == d.N && it->second.K == d.K)
+            prep = &it->second;
+    }
     const long b_batches = d.sB != 0 ? d.G : 1;
     if (kmajor && !d.b32 && d.M > 32 && b_batches * d.N * d.K <= kBRowsMaxElements &&
         (double)d.G * d.M * d.N * d.K >= (getenv("ZK_B_ROWS_MIN_MACS") ? atof(getenv("ZK_B_ROWS_MIN_MACS")) : (double)kBRowsMinMacs)) {
@@ -275,7 +410,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
 
     // (a divided B has another range than the raw one: the shift is part of its key)
     const OperandKey key_a(d.A, (long)d.G * d.M, d.K, 8), key_b(d.B, d.N, d.K, (d.b32 ? 4 : 8) | (b_shift << 8));
-    int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
+    int na = g_cache.lookup(key_a), nb = prep ? prep->nb : g_cache.lookup(key_b);
     // Activations gathered into a fresh buffer for a known weight matrix (the experts of a MoE layer): guess the
     // digits the last activations multiplied with that matrix needed.  A wrong guess costs one guarded recomputation.
     if (!na && nb) {
@@ -298,12 +433,21 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (!na) na = limbs_needed(r[0], r[1]);
         if (!nb) nb = limbs_needed(r[2], r[3]);
     }
+    if (prep) { p.B = prep->planes; p.b_nsub = prep->nsub; p.b_ksteps = prep->ksteps; }
 
     for (int attempt = 0; attempt < 3; attempt++) {
         // the stored bits are [shift, shift + 64) of the sum (the remainder lies below them)
         const int need_diag = (d.shift + 64 + 7) / 8;
-        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
-        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag);
+        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag, prep ? prep->nb : 0, prep ? kB64FlyBPlanes : -1) : nullptr;
+        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag, prep ? prep->nb : 0, prep ? kB64PlanesBoth : -1);
+        if (!inst && prep) {
+            // no kernel with exactly the planes' digit count covers A: this call splits the original B like any other
+            // (nb, the planes' count, covers B)
+            prep = nullptr;
+            p.B = d.B;
+            inst = d.M <= 32 ? pick_instance(na, nb, false, true, need_diag) : nullptr;
+            if (!inst) inst = pick_instance(na, nb, false, false, need_diag);
+        }
         if (!inst) return false;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
@@ -322,9 +466,10 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (total > 0x7FFFFFFFL / 8) return false;
         // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass (never for the
         // 32-row tiles: splitting a handful of rows on the fly is cheaper than another kernel in front)
-        const bool use_planes = !kmajor && p.tiles_n >= 4 && !inst->skinny;
+        const bool use_planes = !kmajor && (p.tiles_n >= 4 || prep) && !inst->skinny;
         if (b_shift && (kmajor || !inst->skinny)) return false;
-        const int variant = b_shift ? (d.b32 ? kB32FlyRs : kB64FlyRs)
+        const int variant = prep ? (inst->skinny ? kB64FlyBPlanes : kB64PlanesBoth)
+                          : b_shift ? (d.b32 ? kB32FlyRs : kB64FlyRs)
                           : kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
@@ -406,6 +551,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
+        g_last_prepared = prep ? 1 : 0;
         {
             const hipError_t err = hipGetLastError();
             if (err != hipSuccess) {
@@ -438,7 +584,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         }
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
-        const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
+        const int need_a = limbs_needed(r[0], r[1]), need_b = prep ? prep->nb : limbs_needed(r[2], r[3]);
         g_cache.store_pair(key_a, need_a, key_b, need_b);
         if (need_a <= inst->na && need_b <= inst->nb) return true;
         na = need_a;
@@ -466,17 +612,38 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
 
     // digits: what these operands needed last time, else the widest the 32-row kernels have
     const OperandKey key_a(d.A, (long)d.rows, d.K, 8), key_b(d.B, (long)d.groups * d.N, d.K, d.b32 ? 4 : 8);
-    int na = g_cache.lookup(key_a), nb = g_cache.lookup(key_b);
+    // the experts' weights prepared beforehand (the table pointer is the key): planes instead of B, an exact digit count
+    const PreparedB *prep = nullptr;
+    {
+        auto it = g_prepared.find((const void *)d.B);
+        if (it != g_prepared.end() && it->second.groups == d.groups && !d.b32 && it->second.N == d.N && it->second.K == d.K)
+            prep = &it->second;
+    }
+    if (prep) { p.grp_b = prep->table; p.b_nsub = prep->nsub; p.b_ksteps = prep->ksteps; }
+    int na = g_cache.lookup(key_a), nb = prep ? prep->nb : g_cache.lookup(key_b);
+    bool na_guessed = false;
     if (!na) {
         auto it = g_cache.partner_a.find(key_b);
         na = it != g_cache.partner_a.end() ? it->second : 5;
+        na_guessed = true;
     }
     if (!nb) nb = 5;
 
     for (int attempt = 0; attempt < 3; attempt++) {
-        const Instance *inst = pick_instance(na, nb, d.b32 != 0, true);
+        const Instance *inst = nullptr;
+        for (int tries = 0; tries < 2 && !inst; tries++) {
+            inst = pick_instance(na, nb, d.b32 != 0, true, 16, prep ? prep->nb : 0, prep ? kB64GroupBPlanes : -1);
+            if (!inst && prep && (inst = pick_instance(na, nb, false, true)) != nullptr) {
+                // no kernel with exactly the planes' digit count covers A: this call splits the original weights
+                prep = nullptr;
+                p.grp_b = d.B;
+            }
+            // a guess taken over from other activations that no 32-row kernel covers: try the widest they have (the
+            // digit check settles it, and the guess would otherwise never be replaced)
+            if (!inst && na_guessed && na > 5) na = 5; else break;
+        }
         if (!inst) return 1;
-        MfmaKernel fn = inst->fn[d.b32 ? kB32Group : kB64Group];
+        MfmaKernel fn = inst->fn[prep ? kB64GroupBPlanes : (d.b32 ? kB32Group : kB64Group)];
         if (!fn) return 1;
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
         const int ksteps = (d.K + 31) / 32;
@@ -499,6 +666,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
+        g_last_prepared = prep ? 1 : 0;
         {
             const hipError_t err = hipGetLastError();
             if (err != hipSuccess) {
@@ -510,13 +678,14 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         range_fold_kernel<<<dim3((unsigned)fold.parts), 256, 0, 0>>>(fold);
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "grouped gemm: range readback failed"); return -1; }
-        const int need_a = limbs_needed(r[0], r[1]), need_b = limbs_needed(r[2], r[3]);
+        const int need_a = limbs_needed(r[0], r[1]), need_b = prep ? prep->nb : limbs_needed(r[2], r[3]);
         g_cache.store_pair(key_a, need_a, key_b, need_b);
         *limbs_a = inst->na;
         *limbs_b = inst->nb;
         if (need_a <= inst->na && need_b <= inst->nb) return 0;
         na = need_a;
         nb = need_b;
+        na_guessed = false;
     }
     set_error(kLaunchFailure, "grouped gemm: digit count did not settle");
     return -1;

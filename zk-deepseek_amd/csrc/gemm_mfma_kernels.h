@@ -36,6 +36,7 @@ struct MfmaParams {
     int verify_b_all_batches;       // B differs per batch: every batch's first tile row tracks its range
     const unsigned char *a_planes;  // pre-split digits of A (planes variants only)
     int a_msub, a_ksteps;           // 32-row groups and 32-k steps the planes were written for
+    int b_nsub, b_ksteps;           // BPL kernels: B (or every group's B) is digit planes of that geometry, prepared beforehand
     // split-K tail: workgroup ids below main_tiles are whole tiles; the rest are `split` workgroups per tile that
     // each cover a slice of K and leave raw 128-bit partial sums in `partials`
     int main_tiles, split;
@@ -395,12 +396,15 @@ __host__ __device__ constexpr int kept_pairs_before(int na, int nb, int d, int i
 // ---- the GEMM kernel -------------------------------------------------------------------------------
 // WVM x WVN waves per workgroup, WM x WN 32x32 MFMA tiles per wave, KK MFMA k-depths (32 k each) per pipeline
 // step.  APL: A comes from pre-split digit planes (plain copy into LDS); otherwise it is split on the fly like B.
+// BPL: so does B (weights prepared once, in the layout of the A planes with columns for rows); nothing of B is tracked then,
+// its digit count was fixed exactly when the planes were made.
 //
 // The hot loop is branch-free: rows past M or N are clamped to the last valid row (their products land in
 // outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
 // own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
 // to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
-template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false, int DMAX = 16>
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false, int DMAX = 16,
+          bool BPL = false>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 {
     constexpr int T = 64 * WVM * WVN;
@@ -472,7 +476,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     // than its neighbours and every element is still seen once.
     const int vmod_b = p.tiles_m < 8 ? p.tiles_m : 8, vmod_a = p.tiles_n < 8 ? p.tiles_n : 8;
     const bool verify_a = !APL && tn < vmod_a;
-    const bool verify_b = tm < vmod_b && (g == 0 || p.verify_b_all_batches);
+    const bool verify_b = !BPL && tm < vmod_b && (g == 0 || p.verify_b_all_batches);
     MinMax ra = { INT64_MAX, INT64_MIN }, rb = { INT64_MAX, INT64_MIN };
     int rb32_lo = INT32_MAX, rb32_hi = INT32_MIN;        // the range of an int32 B is tracked in 32 bits and joins rb at the end
 
@@ -488,23 +492,26 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 
     // Work items of the loaders: (row, j) pairs owning 8 elements each, or 16-byte chunks of digit planes.
     constexpr int A_ITEMS = BM * OCTS, B_ITEMS = BN * OCTS;
-    constexpr int A_IT = APL ? 1 : (A_ITEMS + T - 1) / T, B_IT = (B_ITEMS + T - 1) / T;
+    constexpr int A_IT = APL ? 1 : (A_ITEMS + T - 1) / T, B_IT = BPL ? 1 : (B_ITEMS + T - 1) / T;
     constexpr int A_CHUNKS = KK * A_BLOCKS * 64, A_CIT = APL ? (A_CHUNKS + T - 1) / T : 1;
+    constexpr int B_CHUNKS = KK * B_BLOCKS * 64, B_CIT = BPL ? (B_CHUNKS + T - 1) / T : 1;
+    static_assert(!BPL || (!B32 && !BKM && !BRS && KK == 1), "prepared planes of B: int64 rows, one MFMA depth per step");
     int64_t sa[A_IT][8], sb[B_IT][8];
-    v4i pa[A_CIT];
+    v4i pa[A_CIT], pb[B_CIT];
 
     const bool a_vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
-    const bool b_vec = !BKM && (((uintptr_t)b_base | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
+    const bool b_vec = BPL || !BKM && (((uintptr_t)b_base | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
 
     // per-thread source pointers (advanced by BK per step) and LDS destinations
     const int64_t *a_src[A_IT];
     const unsigned char *a_pl[A_CIT];
     const char *b_src[B_IT];
+    const unsigned char *b_pl[B_CIT];
     // LDS destinations are stage-relative; threads with no work in an iteration aim at a dummy area behind the two
     // stages (and a zero stage stride), which keeps the loop body free of branches.
     constexpr int DUMMY = 2 * STAGE;
-    int a_j[A_IT], b_j[B_IT], a_dst[A_IT], b_dst[B_IT], pl_dst[A_CIT];
-    int a_stride[A_IT], b_stride[B_IT], pl_stride[A_CIT];
+    int a_j[A_IT], b_j[B_IT], a_dst[A_IT], b_dst[B_IT], pl_dst[A_CIT], plb_dst[B_CIT];
+    int a_stride[A_IT], b_stride[B_IT], pl_stride[A_CIT], plb_stride[B_CIT];
     if (APL) {
 #pragma unroll
         for (int it = 0; it < A_CIT; it++) {
@@ -532,8 +539,24 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
             a_stride[it] = live ? STAGE : 0;
         }
     }
+    if (BPL) {
 #pragma unroll
-    for (int it = 0; it < B_IT; it++) {
+        for (int it = 0; it < B_CIT; it++) {
+            const int c = it * T + tid;
+            const bool live = B_CHUNKS % T == 0 || c < B_CHUNKS;
+            const int cc0 = live ? c : 0;
+            // as for the planes of A: LDS order inside a stage is [kk][sub][digit], planes are [sub][ks32][digit]
+            const int kk = cc0 / (B_BLOCKS * 64), cc = cc0 - kk * (B_BLOCKS * 64);
+            const int sub_i = cc / (NB * 64), within = cc - sub_i * (NB * 64);
+            int sub = (n0 >> 5) + sub_i;
+            sub = sub < p.b_nsub ? sub : p.b_nsub - 1;          // column groups past N: any valid data, never stored
+            b_pl[it] = reinterpret_cast<const unsigned char *>(b_base) + ((long)sub * p.b_ksteps + kk) * (NB * 1024) + within * 16;
+            plb_dst[it] = live ? A_BLOCKS * 1024 + kk * SUBSTAGE + cc * 16 : DUMMY;
+            plb_stride[it] = live ? STAGE : 0;
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
         const int idx = it * T + tid;
         const bool live = B_ITEMS % T == 0 || idx < B_ITEMS;
         const int idx0 = live ? idx : 0;
@@ -563,8 +586,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                 else load_owned_i64<RUN, OCTS>(a_src[it] + k0, a_j[it], true, p.K - k0, false, sa[it]);
             }
         }
+        if (BPL) {
 #pragma unroll
-        for (int it = 0; it < B_IT; it++) {
+            for (int it = 0; it < B_CIT; it++)
+                pb[it] = *reinterpret_cast<const v4i *>(b_pl[it] + (long)ks * (KK * NB * 1024));
+        }
+#pragma unroll
+        for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
             if (BKM) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -604,8 +632,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                     *reinterpret_cast<uint2 *>(smem + a_dst[it] + buf * a_stride[it] + i * 1024) = dg[i];
             }
         }
+        if (BPL) {
 #pragma unroll
-        for (int it = 0; it < B_IT; it++) {
+            for (int it = 0; it < B_CIT; it++)
+                *reinterpret_cast<v4i *>(smem + plb_dst[it] + buf * plb_stride[it]) = pb[it];
+        }
+#pragma unroll
+        for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
             uint2 dg[NB];
             if (BRS) {
                 int64_t y[8];
@@ -894,7 +927,8 @@ typedef void (*MfmaKernel)(MfmaParams);
 typedef void (*FinishKernel)(MfmaParams, FoldArgs);
 typedef void (*PlanesKernel)(MfmaParams, unsigned char *, int, int, unsigned long long *);
 
-enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kB64FlyRs, kB32FlyRs, kVariants };
+enum Variant { kB64Fly = 0, kB64Planes, kB32Fly, kB32Planes, kB64KmajorFly, kB32KmajorFly, kB64Group, kB32Group, kB64FlyRs, kB32FlyRs,
+               kB64PlanesBoth, kB64FlyBPlanes, kB64GroupBPlanes, kVariants };     // the last three: B from prepared digit planes
 
 struct Instance {
     int na, nb, bm, bn, threads, kk;
@@ -932,6 +966,12 @@ static Instance make_instance()
         s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX>;
         s.fn[kB64KmajorFly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, true, false, false, false, DMAX>;
     }
+    if constexpr (!B32ONLY && KK == 1 && !SKINNY)
+        s.fn[kB64PlanesBoth] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX, true>;
+    if constexpr (!B32ONLY && KK == 1 && SKINNY) {
+        s.fn[kB64FlyBPlanes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, false, DMAX, true>;
+        s.fn[kB64GroupBPlanes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX, true>;
+    }
     if constexpr (NB <= 5) {          // int32 values never need more than five digits
         s.fn[kB32Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, false, false, false, DMAX>;
         s.fn[kB32Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, false, true, false, false, DMAX>;
@@ -956,5 +996,6 @@ void mfma_instances_mid(std::vector<Instance> &out);
 void mfma_instances_wide(std::vector<Instance> &out);
 void mfma_instances_pruned(std::vector<Instance> &out);
 void mfma_instances_rows32(std::vector<Instance> &out);
+void mfma_instances_rows32b(std::vector<Instance> &out);
 
 }  // namespace zk

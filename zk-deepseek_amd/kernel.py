@@ -57,6 +57,8 @@ lib.wkv_b_bf16_to_int32.argtypes = [_vp, _vp, _ci, _ci]
 lib.fp8_block_scaled_to_int32.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci]
 lib.bf16_scaled_round_to_int32.argtypes = [_vp, _vp, ctypes.c_long, _ci]
 lib.bf16_scaled_round_to_int64.argtypes = [_vp, _vp, ctypes.c_long, _ci]
+lib.zk_gemm_prepare_weights.argtypes = [_vp, _ci, _ci, _ci]
+lib.zk_gemm_release_weights.argtypes = [_vp]
 # additions without a reference counterpart
 lib.rms_stat_int64.argtypes = [_vp, _vp, _ci, _ci, _ll, _ll]
 lib.rms_norm_fused_32.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ll, _ll]
@@ -93,6 +95,22 @@ def _check(what):
         msg = lib.zk_last_error_string().decode()
         lib.zk_clear_error()
         raise RuntimeError("%s failed (code %d): %s" % (what, code, msg))
+
+
+def prepare_weights(W, groups=0, N=None, K=None):
+    """Split an int64 weight matrix [N,K] (or, with groups > 0, every matrix of the device pointer table `W` made by
+    pointer_table) into digit planes once; later int64_bmm_broadcast / int64_grouped_bmm calls with the same tensor
+    read the planes instead of splitting the weights in every tile.  The weights must not change until release_weights."""
+    assert W.is_cuda and W.dtype == torch.int64 and W.is_contiguous()
+    if groups == 0:
+        assert W.dim() == 2
+        N, K = W.shape
+    if lib.zk_gemm_prepare_weights(W.data_ptr(), int(groups), int(N), int(K)) != 0:
+        _check("prepare_weights")
+
+
+def release_weights(W):
+    lib.zk_gemm_release_weights(W.data_ptr())
 
 
 def gemm_last_pairs():
