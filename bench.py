@@ -352,6 +352,21 @@ def main():
                 hbm(nm, lambda: K.moe_experts(xt, wt, it, tabs[0], tabs[1], tabs[2], True, 2048, 30, 33), 1, bytes_per_elem=wbytes, steps=3)
                 extra[nm]["weight_bytes"] = wbytes
                 extra[nm]["experts_hit"] = hit
+            # 256 tokens again with the int32 weights prepared as digit planes (four bytes per weight, as before, but
+            # nothing of B is split in the kernel)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for tb in tabs:
+                K.prepare_weights(tb, groups=256, N=int(2048 if tb is not tabs[2] else 7168), K=int(7168 if tb is not tabs[2] else 2048), b32=True)
+            prep_ms = (time.perf_counter() - t0) * 1e3
+            hit = int(torch.unique(im).numel())
+            wbytes = 3.0 * hit * 2048 * 7168 * 4
+            nm = "moe_experts_int32_256tok_prepared_weights"
+            hbm(nm, lambda: K.moe_experts(xm, wm, im, tabs[0], tabs[1], tabs[2], True, 2048, 30, 33), 1, bytes_per_elem=wbytes, steps=3)
+            extra[nm]["weight_bytes"] = wbytes
+            extra[nm]["prepare_once_ms"] = prep_ms
+            for tb in tabs:
+                K.release_weights(tb)
             del ew1, ew3, ew2, tabs
             torch.cuda.empty_cache()
 

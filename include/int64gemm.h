@@ -201,16 +201,16 @@ int zk_gemm_last_pairs(void);
 long zk_gemm_guard_hits(void);
 /* How many int64_grouped_bmm_launcher calls so far ran as ONE launch over all groups (the others went group by group). */
 long zk_gemm_grouped_mfma_calls(void);
-/* No reference counterpart: model weights do not change between calls, so an int64 weight matrix W[N,K] (groups == 0,
- * B = the device pointer later passed as B) or all the matrices of a device table of pointers (groups > 0, B = the
- * table later passed to int64_grouped_bmm_launcher) can be split into base-256 digit planes ONCE.  Later calls of
- * int64_64_bmm_broadcast_launcher / int64_grouped_bmm_launcher with that pointer, these N and K, b_rescale 1 and
- * contiguous rows then read the planes (as many bytes per weight as its values need digits, 3 for |w| < 2^23, instead
- * of 8) and split nothing of B; results are the same bits.  The library allocates the planes and keeps them until
- * zk_gemm_release_weights or the end of the process.  The original weights must stay where they are and unchanged
- * meanwhile (the exact fallback path reads them).  Returns 0 on success; an error is recorded otherwise.  Waits for
- * the device.  int32 weights are not taken (their planes would be no smaller than they are). */
-int zk_gemm_prepare_weights(const void *B, int groups, int N, int K);
+/* No reference counterpart: model weights do not change between calls, so a weight matrix W[N,K] (int64, or int32 with
+ * b32 != 0; groups == 0, B = the device pointer later passed as B) or all the matrices of a device table of pointers
+ * (groups > 0, B = the table later passed to int64_grouped_bmm_launcher) can be split into base-256 digit planes ONCE.
+ * Later calls of int64_64/32_bmm_broadcast_launcher / int64_grouped_bmm_launcher with that pointer, these N and K,
+ * b_rescale 1 and contiguous rows then read the planes (as many bytes per weight as its values need digits: 3 for
+ * |w| < 2^23, 4 up to 31 bits, else 5 or 9) and split nothing of B; results are the same bits.  The library allocates
+ * the planes and keeps them until zk_gemm_release_weights or the end of the process.  The original weights must stay
+ * where they are and unchanged meanwhile (the exact fallback path and the matrix-vector kernels read them).  Returns 0
+ * on success; an error is recorded otherwise.  Waits for the device. */
+int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K);
 void zk_gemm_release_weights(const void *B);
 /* 1 when the last GEMM-like call ran on the MFMA path and read B from prepared planes, else 0. */
 int zk_gemm_last_prepared(void);

@@ -171,9 +171,25 @@ def test_config5_decoder_layer_full_size(backends):
     # the same layer through the fused entry points and the device-side MoE (routing, dispatch, ONE grouped launch per
     # expert matrix over all 256 experts, combine): identical output
     before = kernel.lib.zk_gemm_grouped_mfma_calls()
-    y2, idx2 = H.decoder_layer(H.FusedGpuBackend(kernel), x, P, freqs, cfg)
+    fused = H.FusedGpuBackend(kernel)
+    y2, idx2 = H.decoder_layer(fused, x, P, freqs, cfg)
     assert kernel.lib.zk_gemm_grouped_mfma_calls() - before == 3
     assert np.array_equal(idx2, idx) and torch.equal(y2, y)
+    # and once more with every int64 weight matrix prepared as digit planes (the expert tables and the linears):
+    # identical output again, the experts' launches read the planes
+    prepared = []
+    for tab, (n, k) in zip(fused._tables, ((inter, dim), (inter, dim), (dim, inter))):
+        kernel.prepare_weights(tab, groups=E, N=n, K=k)
+        prepared.append(tab)
+    for name in ("wq_a", "wq_b1", "wq_b2", "wkv_a1", "wkv_a2", "wo", "gate", "sw1", "sw3", "sw2"):
+        kernel.prepare_weights(P[name])
+        prepared.append(P[name])
+    before = kernel.lib.zk_gemm_grouped_mfma_calls()
+    y3, idx3 = H.decoder_layer(fused, x, P, freqs, cfg)
+    assert kernel.lib.zk_gemm_grouped_mfma_calls() - before == 3
+    assert np.array_equal(idx3, idx) and torch.equal(y3, y)
+    for t in prepared:
+        kernel.release_weights(t)
     # the layer's output is alive: neither stuck at the residual nor saturated
     d = (y - x).abs()
     assert int(d.max()) > 0 and int(y.abs().max()) < 1 << 62

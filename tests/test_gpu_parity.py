@@ -231,16 +231,17 @@ def test_gemm_rows_staged_in_lds(K, oracle, M):
     assert K.gemm_last_plan()[0] == 1
 
 
-@pytest.mark.parametrize("bits_w", [16, 28, 36, 63])
+@pytest.mark.parametrize("bits_w", [16, 28, 36, 63, -16, -30, -31])
 def test_gemm_prepared_weights(K, oracle, bits_w):
     """int64 weights split into digit planes once (zk_gemm_prepare_weights): the same bits as the unprepared call on
     32-row and full tiles, ragged N and K, split K, few rows, activations that need more digits than any kernel with the
     planes' digit count has (the call then splits the original weights), weights changed and prepared again, release"""
-    rng = np.random.default_rng(bits_w)
+    w32, bits_w = bits_w < 0, abs(bits_w)                # negative: int32 weights of that many bits
+    rng = np.random.default_rng(bits_w + w32)
     for M, Kd, N, bits_a, c in ((16, 7168, 576, 20, 29), (130, 300, 150, 20, 0), (512, 1000, 700, 23, 29), (3, 333, 77, 30, 33),
                                 (1, 520, 300, 20, 23), (70, 96, 2100, 63, 31)):
         A = rand_i64(rng, (2, M, Kd), bits_a)
-        W = rand_i64(rng, (N, Kd), bits_w)
+        W = rand_i32(rng, (N, Kd), bits_w) if w32 else rand_i64(rng, (N, Kd), bits_w)
         W[0, :2] = [-(1 << bits_w), (1 << bits_w) - 1]
         Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, c)
         Ad, Wd = dev(A), dev(W)
@@ -251,7 +252,7 @@ def test_gemm_prepared_weights(K, oracle, bits_w):
         if bits_a <= 23 and bits_w <= 36 and M > 4:
             assert K.lib.zk_gemm_last_prepared() == 1            # the planes were used
         # other weights under the same pointer, prepared again
-        W2 = rand_i64(rng, (N, Kd), 12)
+        W2 = rand_i32(rng, (N, Kd), 12) if w32 else rand_i64(rng, (N, Kd), 12)
         Wd.copy_(dev(W2))
         K.prepare_weights(Wd)
         C, R = K.int64_bmm_broadcast(Ad, Wd, 1, 1, c)
@@ -263,17 +264,18 @@ def test_gemm_prepared_weights(K, oracle, bits_w):
         assert K.lib.zk_gemm_last_prepared() == 0
 
 
+@pytest.mark.parametrize("w32", [False, True])
 @pytest.mark.parametrize("T,Kr", [(1, 8), (40, 3), (300, 4)])
-def test_grouped_bmm_prepared_weights(K, oracle, T, Kr):
+def test_grouped_bmm_prepared_weights(K, oracle, T, Kr, w32):
     """the experts' weights prepared through their pointer table: one launch over all experts on the planes, the same
     bits as without; wide activations fall back to splitting the original weights"""
     rng = np.random.default_rng(T + Kr)
     E, Kd, N = 16, 200, 300
     idx = _routing(rng, T, E, Kr)
-    ws = [rand_i64(rng, (N, Kd), 16) for _ in range(E)]
+    ws = [rand_i32(rng, (N, Kd), 30) if w32 else rand_i64(rng, (N, Kd), 16) for _ in range(E)]
     wd = [dev(w) for w in ws]
     tab = K.pointer_table(wd)
-    K.prepare_weights(tab, groups=E, N=N, K=Kd)
+    K.prepare_weights(tab, groups=E, N=N, K=Kd, b32=w32)
     d = K.moe_dispatch(dev(idx), E)
     seg, tok, _ = oracle.moe_dispatch(idx, E)
     for bits_a in (20, 45):
@@ -281,14 +283,14 @@ def test_grouped_bmm_prepared_weights(K, oracle, T, Kr):
         xs = K.moe_gather_rows(dev(x), d)
         before = K.lib.zk_gemm_grouped_mfma_calls()
         for c in (0, 19):
-            C, R = K.int64_grouped_bmm(xs, tab, False, N, c, d, want_remainder=True)
+            C, R = K.int64_grouped_bmm(xs, tab, w32, N, c, d, want_remainder=True)
             Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
             assert np.array_equal(host(C), Ce), ("quotient", bits_a, c)
             assert np.array_equal(host(R), Re), ("remainder", bits_a, c)
-        if bits_a == 20 and T * Kr > 32:
+        if bits_a == 20 and T * Kr > (64 if w32 else 32):
             assert K.lib.zk_gemm_grouped_mfma_calls() - before == 2 and K.lib.zk_gemm_last_prepared() == 1
     K.release_weights(tab)
-    C = K.int64_grouped_bmm(xs, tab, False, N, 19, d)
+    C = K.int64_grouped_bmm(xs, tab, w32, N, 19, d)
     assert np.array_equal(host(C), oracle.grouped_bmm(x[tok], ws, seg, 19)[0])
 
 

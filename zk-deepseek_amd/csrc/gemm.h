@@ -41,8 +41,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 // Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
 // vector-ALU recomputation (known once their range has reached the host).
 long gemm_mfma_guard_hits();
-// weights prepared once as digit planes (int64 matrices, or a device table of `groups` of them): 0 on success
-int gemm_mfma_prepare(const void *B, int groups, int N, int K);
+// weights prepared once as digit planes (an int64 or int32 matrix, or a device table of `groups` of them): 0 on success
+int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K);
 void gemm_mfma_release(const void *B);
 bool gemm_mfma_is_prepared(const void *B);
 int gemm_mfma_last_pairs();

@@ -18,7 +18,7 @@ void gemm_dispatch(const char *name, const GemmDesc &d)
     // (prepared weights: the MFMA kernels read a few bytes per weight where the matrix-vector stream reads eight, so
     // from 128 MB of weights on they go first and the matrix-vector kernels only if the MFMA path does not take the
     // product.  One row against [18432,7168]: 0.19 -> 0.087 ms; against [576,7168] the stream wins, 9 against 22 us.)
-    const bool prepared = g_gemm_path != kPathValu && (long)d.N * d.K >= (16L << 20) && gemm_mfma_is_prepared(d.B);
+    const bool prepared = g_gemm_path != kPathValu && !d.b32 && (long)d.N * d.K >= (16L << 20) && gemm_mfma_is_prepared(d.B);
     if (g_gemm_path != kPathMfma && !prepared && gemm_gemv_launch(d)) {
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
         check_launch(name);
@@ -53,7 +53,7 @@ void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
 {
     // (prepared weights: from 33 rows on the MFMA kernels first, as in gemm_dispatch; below that the handful of tiles
     // leaves most of the device idle and the row-by-row stream is faster: one token 0.52 against 0.66 ms)
-    const bool prepared = g_gemm_path != kPathValu && d.rows > 32 && gemm_mfma_is_prepared((const void *)d.B);
+    const bool prepared = g_gemm_path != kPathValu && !d.b32 && d.rows > 32 && gemm_mfma_is_prepared((const void *)d.B);
     const bool few_rows = g_gemm_path != kPathMfma && d.rows <= kGroupedGemvMaxRows && d.K > 0;
     if (few_rows && !prepared && gemm_gemv_grouped_launch(d)) {
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
@@ -232,7 +232,7 @@ int zk_gemm_last_pairs(void) { return zk::g_last_path == zk::kPathMfma ? zk::gem
 long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
 
 int zk_gemm_last_prepared(void) { return zk::g_last_path == zk::kPathMfma ? zk::gemm_mfma_last_prepared() : 0; }
-int zk_gemm_prepare_weights(const void *B, int groups, int N, int K) { return zk::gemm_mfma_prepare(B, groups, N, K); }
+int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K) { return zk::gemm_mfma_prepare(B, b32, groups, N, K); }
 void zk_gemm_release_weights(const void *B) { zk::gemm_mfma_release(B); }
 
 }  // extern "C"

@@ -224,14 +224,15 @@ static FoldArgs make_fold(const unsigned long long *mm, long mm_count, const uns
 struct PreparedB {
     unsigned char *planes = nullptr;     // per matrix: [nsub][ksteps][nb] blocks of 1 KB
     const void **table = nullptr;        // device array: the planes of every group (tables only)
-    int groups = 0, N = 0, K = 0, nb = 0, nsub = 0, ksteps = 0;
+    int groups = 0, N = 0, K = 0, nb = 0, nsub = 0, ksteps = 0, b32 = 0;
 };
 static std::map<const void *, PreparedB> g_prepared;
 
-static __global__ __launch_bounds__(256) void range_exact_kernel(const int64_t *__restrict__ x, long n, unsigned long long *out)
+template <typename T>
+static __global__ __launch_bounds__(256) void range_exact_kernel(const T *__restrict__ x, long n, unsigned long long *out)
 {
     MinMax r = { INT64_MAX, INT64_MIN };
-    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) mm_update(r, x[i]);
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) mm_update(r, (int64_t)x[i]);
     r = mm_wave(r);
     if ((threadIdx.x & 63) == 0 && r.lo <= r.hi) {
         atomicMin(out, (unsigned long long)r.lo ^ kSignFlip);
@@ -262,7 +263,7 @@ void gemm_mfma_release(const void *B)
     g_prepared.erase(it);
 }
 
-int gemm_mfma_prepare(const void *B, int groups, int N, int K)
+int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
 {
     const char *name = "zk_gemm_prepare_weights";
     if (!B || groups < 0 || groups > 65535 || N < 1 || K < 1) { set_error(kBadArgument, "%s: bad argument", name); return 1; }
@@ -284,13 +285,15 @@ int gemm_mfma_prepare(const void *B, int groups, int N, int K)
     const long elems = (long)N * K;
     range_reset_kernel<<<1, 64, 0, 0>>>(g_cache.dev);
     const unsigned rgrid = (unsigned)(elems / 256 + 1 < 2048 ? elems / 256 + 1 : 2048);
-    for (int i = 0; i < count; i++)
-        range_exact_kernel<<<rgrid, 256, 0, 0>>>(reinterpret_cast<const int64_t *>(mats[i]), elems, g_cache.dev);
+    for (int i = 0; i < count; i++) {
+        if (b32) range_exact_kernel<int32_t><<<rgrid, 256, 0, 0>>>(reinterpret_cast<const int32_t *>(mats[i]), elems, g_cache.dev);
+        else range_exact_kernel<int64_t><<<rgrid, 256, 0, 0>>>(reinterpret_cast<const int64_t *>(mats[i]), elems, g_cache.dev);
+    }
     int64_t r[4];
     if (!read_range(g_cache.dev, r)) { set_error(kLaunchFailure, "%s: range readback failed", name); return 1; }
     const int need = limbs_needed(r[0], r[1]);
     PreparedB pb;
-    pb.groups = groups; pb.N = N; pb.K = K;
+    pb.groups = groups; pb.N = N; pb.K = K; pb.b32 = b32 ? 1 : 0;
     pb.nb = need <= 3 ? 3 : (need <= 5 ? need : 9);              // digit counts the kernels are built for
     pb.nsub = (N + 31) / 32;
     pb.ksteps = (K + 31) / 32;
@@ -319,12 +322,15 @@ int gemm_mfma_prepare(const void *B, int groups, int N, int K)
     for (int i = 0; i < count; i++) {
         q.A = reinterpret_cast<const int64_t *>(mats[i]);
         unsigned char *dst = pb.planes + per * i;
+#define ZK_PLANES(NB_) do { if (b32) a_planes_kernel<NB_, 2, 1, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); \
+                           else a_planes_kernel<NB_, 2, 1, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); } while (0)
         switch (pb.nb) {
-        case 3: a_planes_kernel<3, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
-        case 4: a_planes_kernel<4, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
-        case 5: a_planes_kernel<5, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
-        default: a_planes_kernel<9, 2, 1><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); break;
+        case 3: ZK_PLANES(3); break;
+        case 4: ZK_PLANES(4); break;
+        case 5: ZK_PLANES(5); break;
+        default: ZK_PLANES(9); break;
         }
+#undef ZK_PLANES
     }
     if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
         release_prepared(pb);
@@ -386,8 +392,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     const PreparedB *prep = nullptr;
     {
         auto it = g_prepared.find(d.B);
-        if (it != g_prepared.end() && it->second.groups == 0 && !d.b32 && !kmajor && b_shift == 0 && d.sB == 0 && d.ldbk == 1 &&
-            d.ldbn == d.K && it->second.N == d.N && it->second.K == d.K)
+        if (it != g_prepared.end() && it->second.groups == 0 && it->second.b32 == (d.b32 ? 1 : 0) && !kmajor && b_shift == 0 && d.sB == 0 &&
+            d.ldbk == 1 && d.ldbn == d.K && it->second.N == d.N && it->second.K == d.K)
             prep = &it->second;
     }
     const long b_batches = d.sB != 0 ? d.G : 1;
@@ -438,15 +444,16 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     for (int attempt = 0; attempt < 3; attempt++) {
         // the stored bits are [shift, shift + 64) of the sum (the remainder lies below them)
         const int need_diag = (d.shift + 64 + 7) / 8;
-        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag, prep ? prep->nb : 0, prep ? kB64FlyBPlanes : -1) : nullptr;
-        if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag, prep ? prep->nb : 0, prep ? kB64PlanesBoth : -1);
+        // (the kernels that read planes never see B's element type: they are the int64 forms)
+        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0 && !prep, true, need_diag, prep ? prep->nb : 0, prep ? kB64FlyBPlanes : -1) : nullptr;
+        if (!inst) inst = pick_instance(na, nb, d.b32 != 0 && !prep, false, need_diag, prep ? prep->nb : 0, prep ? kB64PlanesBoth : -1);
         if (!inst && prep) {
             // no kernel with exactly the planes' digit count covers A: this call splits the original B like any other
             // (nb, the planes' count, covers B)
             prep = nullptr;
             p.B = d.B;
-            inst = d.M <= 32 ? pick_instance(na, nb, false, true, need_diag) : nullptr;
-            if (!inst) inst = pick_instance(na, nb, false, false, need_diag);
+            inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
+            if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag);
         }
         if (!inst) return false;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
@@ -538,7 +545,8 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)((msub * 32 + rows_per_wg - 1) / rows_per_wg), (unsigned)d.G);
             plane_wgs = (long)pgrid.x * pgrid.y * pgrid.z;
             if (!grow(g_cache.mm, g_cache.mm_count, (size_t)plane_wgs * 2, "range scratch")) return false;
-            inst->planes[d.b32 ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
+            // (the owned-k pattern of the planes of A follows the kernel that reads them: prepared planes of B go with the int64 forms)
+            inst->planes[(d.b32 && !prep) ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
         }
         const size_t lds = 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
         static std::set<const void *> lds_raised;
@@ -616,7 +624,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
     const PreparedB *prep = nullptr;
     {
         auto it = g_prepared.find((const void *)d.B);
-        if (it != g_prepared.end() && it->second.groups == d.groups && !d.b32 && it->second.N == d.N && it->second.K == d.K)
+        if (it != g_prepared.end() && it->second.groups == d.groups && it->second.b32 == (d.b32 ? 1 : 0) && it->second.N == d.N && it->second.K == d.K)
             prep = &it->second;
     }
     if (prep) { p.grp_b = prep->table; p.b_nsub = prep->nsub; p.b_ksteps = prep->ksteps; }
@@ -632,8 +640,8 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
     for (int attempt = 0; attempt < 3; attempt++) {
         const Instance *inst = nullptr;
         for (int tries = 0; tries < 2 && !inst; tries++) {
-            inst = pick_instance(na, nb, d.b32 != 0, true, 16, prep ? prep->nb : 0, prep ? kB64GroupBPlanes : -1);
-            if (!inst && prep && (inst = pick_instance(na, nb, false, true)) != nullptr) {
+            inst = pick_instance(na, nb, d.b32 != 0 && !prep, true, 16, prep ? prep->nb : 0, prep ? kB64GroupBPlanes : -1);
+            if (!inst && prep && (inst = pick_instance(na, nb, d.b32 != 0, true)) != nullptr) {
                 // no kernel with exactly the planes' digit count covers A: this call splits the original weights
                 prep = nullptr;
                 p.grp_b = d.B;

@@ -259,7 +259,8 @@ __device__ __forceinline__ int frag_offset(int row, int j, int n_limbs, int subs
 // block (g, sub, ks32, i) of 1 KB holds digit i of rows [32*sub, 32*sub+32) for the 32 owned-k slots of MFMA
 // depth ks32, lane-major.  Rows >= M and k >= K are written as zero digits.  Each workgroup also leaves the
 // min and max of what it read in mm[2*block .. 2*block+1].
-template <int NA, int RUN, int KK>
+// IN32: the matrix holds int32 elements (weights prepared once; lda and sA count elements as they do for int64).
+template <int NA, int RUN, int KK, bool IN32 = false>
 __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned char *planes, int msub, int ksteps32,
                                                        unsigned long long *mm)
 {
@@ -271,7 +272,8 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
     const int k0 = ks * (8 * OCTS);
     const bool vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
     int64_t x[8];
-    load_owned_i64<RUN, OCTS>(p.A + (long)g * p.sA + (long)row * p.lda + k0, j, row < p.M, p.K - k0, vec, x);
+    if (IN32) load_owned_i32<RUN, OCTS>(reinterpret_cast<const int32_t *>(p.A) + (long)g * p.sA + (long)row * p.lda + k0, j, row < p.M, p.K - k0, false, x);
+    else load_owned_i64<RUN, OCTS>(p.A + (long)g * p.sA + (long)row * p.lda + k0, j, row < p.M, p.K - k0, vec, x);
     MinMax r = { INT64_MAX, INT64_MIN };
 #pragma unroll
     for (int q = 0; q < 8; q++) mm_update(r, x[q]);

@@ -57,7 +57,7 @@ lib.wkv_b_bf16_to_int32.argtypes = [_vp, _vp, _ci, _ci]
 lib.fp8_block_scaled_to_int32.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci]
 lib.bf16_scaled_round_to_int32.argtypes = [_vp, _vp, ctypes.c_long, _ci]
 lib.bf16_scaled_round_to_int64.argtypes = [_vp, _vp, ctypes.c_long, _ci]
-lib.zk_gemm_prepare_weights.argtypes = [_vp, _ci, _ci, _ci]
+lib.zk_gemm_prepare_weights.argtypes = [_vp, _ci, _ci, _ci, _ci]
 lib.zk_gemm_release_weights.argtypes = [_vp]
 # additions without a reference counterpart
 lib.rms_stat_int64.argtypes = [_vp, _vp, _ci, _ci, _ll, _ll]
@@ -97,15 +97,19 @@ def _check(what):
         raise RuntimeError("%s failed (code %d): %s" % (what, code, msg))
 
 
-def prepare_weights(W, groups=0, N=None, K=None):
-    """Split an int64 weight matrix [N,K] (or, with groups > 0, every matrix of the device pointer table `W` made by
-    pointer_table) into digit planes once; later int64_bmm_broadcast / int64_grouped_bmm calls with the same tensor
-    read the planes instead of splitting the weights in every tile.  The weights must not change until release_weights."""
-    assert W.is_cuda and W.dtype == torch.int64 and W.is_contiguous()
+def prepare_weights(W, groups=0, N=None, K=None, b32=False):
+    """Split a weight matrix [N,K] (int64 or int32) or, with groups > 0, every matrix of the device pointer table `W` made
+    by pointer_table (b32 says whether they are int32) into digit planes once; later int64_bmm_broadcast /
+    int64_grouped_bmm calls with the same tensor read the planes instead of splitting the weights in every tile.  The
+    weights must not change until release_weights."""
+    assert W.is_cuda and W.is_contiguous()
     if groups == 0:
-        assert W.dim() == 2
+        assert W.dim() == 2 and W.dtype in (torch.int64, torch.int32)
         N, K = W.shape
-    if lib.zk_gemm_prepare_weights(W.data_ptr(), int(groups), int(N), int(K)) != 0:
+        b32 = W.dtype == torch.int32
+    else:
+        assert W.dtype == torch.int64 and W.numel() == groups
+    if lib.zk_gemm_prepare_weights(W.data_ptr(), 1 if b32 else 0, int(groups), int(N), int(K)) != 0:
         _check("prepare_weights")
 
 
