@@ -48,6 +48,7 @@ static const Instance *instances(int *count)
         mfma_instances_pruned(t);
         mfma_instances_rows32(t);
         mfma_instances_rows32b(t);
+        mfma_instances_rows32c(t);
 #endif
         return t;
     }();
@@ -57,7 +58,7 @@ static const Instance *instances(int *count)
 
 // need_diag: the result's top bit is below 2^(8 need_diag), so diagonals from need_diag up cannot reach it
 // exact_nb / variant: for B from prepared planes the instance must have exactly the planes' digit count and that kernel
-static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int need_diag = 16, int exact_nb = 0, int variant = -1)
+static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int need_diag = 16, int exact_nb = 0, int variant = -1, int exact_kk = 1)
 {
     int count;
     const Instance *t = instances(&count);
@@ -66,10 +67,10 @@ static const Instance *pick_instance(int na, int nb, bool b32, bool skinny, int 
     for (int i = 0; i < count; i++) {
         if (t[i].na < na || t[i].nb < nb || t[i].skinny != skinny) continue;
         if (t[i].dmax < 16 && t[i].dmax < need_diag) continue;
-        if (exact_nb && t[i].nb != exact_nb) continue;
+        if (exact_nb && (t[i].nb != exact_nb || t[i].kk != exact_kk)) continue;
         if (variant >= 0 && !t[i].fn[variant]) continue;
-        if (b32 && !t[i].fn[kB32Fly]) continue;
-        if (!b32 && !t[i].fn[kB64Fly]) continue;
+        if (variant < 0 && b32 && !t[i].fn[kB32Fly]) continue;
+        if (variant < 0 && !b32 && !t[i].fn[kB64Fly]) continue;
         long cost = kept_pairs_before(t[i].na, t[i].nb, t[i].dmax, t[i].na, 0);     // MFMAs per 32x32x32 block
         // at equal MFMA count the deeper step wins (only instances made for int32 B have one)
         if (!best || cost < best_cost || (cost == best_cost && t[i].kk > best->kk)) { best = &t[i]; best_cost = cost; }
@@ -225,6 +226,7 @@ struct PreparedB {
     unsigned char *planes = nullptr;     // per matrix: [nsub][ksteps][nb] blocks of 1 KB
     const void **table = nullptr;        // device array: the planes of every group (tables only)
     int groups = 0, N = 0, K = 0, nb = 0, nsub = 0, ksteps = 0, b32 = 0;
+    int kk = 1;                          // MFMA depths per step of the kernels the planes were ordered for
 };
 static std::map<const void *, PreparedB> g_prepared;
 
@@ -295,8 +297,10 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
     PreparedB pb;
     pb.groups = groups; pb.N = N; pb.K = K; pb.b32 = b32 ? 1 : 0;
     pb.nb = need <= 3 ? 3 : (need <= 5 ? need : 9);              // digit counts the kernels are built for
+    // the experts' three-digit planes go to kernels with two depths per step (the k-order inside a step follows it)
+    pb.kk = (groups > 0 && pb.nb == 3) ? 2 : 1;
     pb.nsub = (N + 31) / 32;
-    pb.ksteps = (K + 31) / 32;
+    pb.ksteps = ((K + 32 * pb.kk - 1) / (32 * pb.kk)) * pb.kk;
     const size_t per = (size_t)pb.nsub * pb.ksteps * pb.nb * 1024;
     if (hipMalloc(&pb.planes, per * count) != hipSuccess) {
         (void)hipGetLastError();
@@ -315,7 +319,8 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
         }
     }
     // the pre-pass that splits A in fragment order does the same for the rows of a weight matrix (64 rows per workgroup)
-    const dim3 grid((unsigned)pb.ksteps, (unsigned)((pb.nsub * 32 + 63) / 64), 1);
+    const int rows_per_wg = 256 / (4 * pb.kk);
+    const dim3 grid((unsigned)(pb.ksteps / pb.kk), (unsigned)((pb.nsub * 32 + rows_per_wg - 1) / rows_per_wg), 1);
     if (!grow(g_cache.mm, g_cache.mm_count, (size_t)grid.x * grid.y * 2, "range scratch")) { release_prepared(pb); return 1; }
     MfmaParams q = {};
     q.lda = K; q.sA = 0; q.M = N; q.K = K;
@@ -325,7 +330,14 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
 #define ZK_PLANES(NB_) do { if (b32) a_planes_kernel<NB_, 2, 1, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); \
                            else a_planes_kernel<NB_, 2, 1, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); } while (0)
         switch (pb.nb) {
-        case 3: ZK_PLANES(3); break;
+        case 3:
+            if (pb.kk == 2) {
+                if (b32) a_planes_kernel<3, 2, 2, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm);
+                else a_planes_kernel<3, 2, 2, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm);
+            } else {
+                ZK_PLANES(3);
+            }
+            break;
         case 4: ZK_PLANES(4); break;
         case 5: ZK_PLANES(5); break;
         default: ZK_PLANES(9); break;
@@ -640,7 +652,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
     for (int attempt = 0; attempt < 3; attempt++) {
         const Instance *inst = nullptr;
         for (int tries = 0; tries < 2 && !inst; tries++) {
-            inst = pick_instance(na, nb, d.b32 != 0 && !prep, true, 16, prep ? prep->nb : 0, prep ? kB64GroupBPlanes : -1);
+            inst = pick_instance(na, nb, d.b32 != 0 && !prep, true, 16, prep ? prep->nb : 0, prep ? kB64GroupBPlanes : -1, prep ? prep->kk : 1);
             if (!inst && prep && (inst = pick_instance(na, nb, d.b32 != 0, true)) != nullptr) {
                 // no kernel with exactly the planes' digit count covers A: this call splits the original weights
                 prep = nullptr;

@@ -497,7 +497,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     constexpr int A_IT = APL ? 1 : (A_ITEMS + T - 1) / T, B_IT = BPL ? 1 : (B_ITEMS + T - 1) / T;
     constexpr int A_CHUNKS = KK * A_BLOCKS * 64, A_CIT = APL ? (A_CHUNKS + T - 1) / T : 1;
     constexpr int B_CHUNKS = KK * B_BLOCKS * 64, B_CIT = BPL ? (B_CHUNKS + T - 1) / T : 1;
-    static_assert(!BPL || (!B32 && !BKM && !BRS && KK == 1), "prepared planes of B: int64 rows, one MFMA depth per step");
+    static_assert(!BPL || (!B32 && !BKM && !BRS), "prepared planes of B go with the int64 forms (and are made for the kernel's KK: the owned-k order depends on it)");
     int64_t sa[A_IT][8], sb[B_IT][8];
     v4i pa[A_CIT], pb[B_CIT];
 
@@ -945,7 +945,8 @@ struct Instance {
 // KKSEL: MFMA k-depths (of 32) per pipeline step.  B32ONLY: an instance for int32 B alone.  The 32-row kernels live on
 // the bytes they keep in flight, and a step of int32 weights is half the bytes of a step of int64 weights: with two
 // depths per step they stream as much per step as the int64 kernels do (where the two LDS stages still fit).
-template <int NA, int NB, bool SKINNY = false, int DMAX = 16, int KKSEL = ZK_KK(0), bool B32ONLY = false>
+// BPLONLY: an instance for grouped launches on prepared planes of B alone (deeper steps for them: more bytes in flight).
+template <int NA, int NB, bool SKINNY = false, int DMAX = 16, int KKSEL = ZK_KK(0), bool B32ONLY = false, bool BPLONLY = false>
 static Instance make_instance()
 {
     constexpr int DD = (NA + NB - 1) > DMAX ? DMAX : (NA + NB - 1);      // diagonals kept = accumulator sets
@@ -963,6 +964,14 @@ static Instance make_instance()
     s.skinny = SKINNY;
     s.dmax = DMAX;
     for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
+    if constexpr (BPLONLY) {
+        static_assert(SKINNY && !B32ONLY, "grouped launches run on the 32-row tiles");
+        s.fn[kB64GroupBPlanes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX, true>;
+        s.finish = gemm_split_finish_kernel<WVM, WVN, WM, WN>;
+        s.planes[0] = a_planes_kernel<NA, 2, KK>;
+        s.planes[1] = a_planes_kernel<NA, 4, KK>;
+        return s;
+    }
     if constexpr (!B32ONLY) {
         s.fn[kB64Fly] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, false, false, DMAX>;
         s.fn[kB64Planes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, true, false, false, DMAX>;
@@ -999,5 +1008,6 @@ void mfma_instances_wide(std::vector<Instance> &out);
 void mfma_instances_pruned(std::vector<Instance> &out);
 void mfma_instances_rows32(std::vector<Instance> &out);
 void mfma_instances_rows32b(std::vector<Instance> &out);
+void mfma_instances_rows32c(std::vector<Instance> &out);
 
 }  // namespace zk
