@@ -234,7 +234,27 @@ template <typename T>
 static __global__ __launch_bounds__(256) void range_exact_kernel(const T *__restrict__ x, long n, unsigned long long *out)
 {
     MinMax r = { INT64_MAX, INT64_MIN };
-    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) mm_update(r, (int64_t)x[i]);
+    // 16-byte pieces, four in flight per thread, then whatever is left (n and the pointer need not be aligned)
+    constexpr int PER = 16 / sizeof(T);
+    const long head = ((uintptr_t)x & 15) ? n : 0;                       // unaligned: everything goes element by element
+    const long pieces = (n - head) / PER;
+    const v4i *xv = reinterpret_cast<const v4i *>(x);
+    for (long q0 = (long)blockIdx.x * 1024 + threadIdx.x; q0 < pieces; q0 += (long)gridDim.x * 1024) {
+        v4i t[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) t[u] = q0 + 256 * u < pieces ? __builtin_nontemporal_load(xv + q0 + 256 * u) : xv[0];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (sizeof(T) == 8) {
+                mm_update(r, (int64_t)(((uint64_t)(uint32_t)t[u][1] << 32) | (uint32_t)t[u][0]));
+                mm_update(r, (int64_t)(((uint64_t)(uint32_t)t[u][3] << 32) | (uint32_t)t[u][2]));
+            } else {
+#pragma unroll
+                for (int z = 0; z < 4; z++) mm_update(r, (int64_t)t[u][z]);
+            }
+        }
+    }
+    for (long i = (head ? 0 : pieces * PER) + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) mm_update(r, (int64_t)x[i]);
     r = mm_wave(r);
     if ((threadIdx.x & 63) == 0 && r.lo <= r.hi) {
         atomicMin(out, (unsigned long long)r.lo ^ kSignFlip);
