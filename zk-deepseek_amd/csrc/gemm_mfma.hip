@@ -49,6 +49,7 @@ static const Instance *instances(int *count)
         mfma_instances_rows32(t);
         mfma_instances_rows32b(t);
         mfma_instances_rows32c(t);
+        mfma_instances_rows32d(t);
 #endif
         return t;
     }();
@@ -317,8 +318,8 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
     PreparedB pb;
     pb.groups = groups; pb.N = N; pb.K = K; pb.b32 = b32 ? 1 : 0;
     pb.nb = need <= 3 ? 3 : (need <= 5 ? need : 9);              // digit counts the kernels are built for
-    // the experts' three-digit planes go to kernels with two depths per step (the k-order inside a step follows it)
-    pb.kk = (groups > 0 && pb.nb == 3) ? 2 : 1;
+    // the experts' three- and four-digit planes go to kernels with two depths per step (the k-order inside a step follows it)
+    pb.kk = (groups > 0 && pb.nb <= 4) ? 2 : 1;
     pb.nsub = (N + 31) / 32;
     pb.ksteps = ((K + 32 * pb.kk - 1) / (32 * pb.kk)) * pb.kk;
     const size_t per = (size_t)pb.nsub * pb.ksteps * pb.nb * 1024;
@@ -350,15 +351,11 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
 #define ZK_PLANES(NB_) do { if (b32) a_planes_kernel<NB_, 2, 1, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); \
                            else a_planes_kernel<NB_, 2, 1, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); } while (0)
         switch (pb.nb) {
-        case 3:
-            if (pb.kk == 2) {
-                if (b32) a_planes_kernel<3, 2, 2, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm);
-                else a_planes_kernel<3, 2, 2, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm);
-            } else {
-                ZK_PLANES(3);
-            }
-            break;
-        case 4: ZK_PLANES(4); break;
+#define ZK_PLANES2(NB_) do { if (b32) a_planes_kernel<NB_, 2, 2, true><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); \
+                            else a_planes_kernel<NB_, 2, 2, false><<<grid, dim3(256), 0, 0>>>(q, dst, pb.nsub, pb.ksteps, g_cache.mm); } while (0)
+        case 3: if (pb.kk == 2) ZK_PLANES2(3); else ZK_PLANES(3); break;
+        case 4: if (pb.kk == 2) ZK_PLANES2(4); else ZK_PLANES(4); break;
+#undef ZK_PLANES2
         case 5: ZK_PLANES(5); break;
         default: ZK_PLANES(9); break;
         }

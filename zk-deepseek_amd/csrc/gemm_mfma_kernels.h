@@ -1009,5 +1009,6 @@ void mfma_instances_pruned(std::vector<Instance> &out);
 void mfma_instances_rows32(std::vector<Instance> &out);
 void mfma_instances_rows32b(std::vector<Instance> &out);
 void mfma_instances_rows32c(std::vector<Instance> &out);
+void mfma_instances_rows32d(std::vector<Instance> &out);
 
 }  // namespace zk
