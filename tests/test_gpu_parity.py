@@ -838,6 +838,37 @@ def test_activation_table_path(K, oracle, fn, Q):
     oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("fn,Q", ACTS)
+def test_activation_quotients_follow_the_table(K, oracle, fn, Q):
+    """the quotients made from the caller's table are kept between calls: a table rewritten in place under the same
+    pointer, and the old table coming back, must show in the very next call and in the calls after it, whether or not
+    the host has waited for the device in between"""
+    rng = np.random.default_rng(300 + Q)
+    n = (1 << 20) + 2
+    x = rng.integers(-(18 << Q), 18 << Q, size=(1, 1, n), dtype=np.int64)
+    default = host(K.EXP2_FRAC_LUT_Q23 if Q == 23 else K.EXP2_FRAC_LUT_Q25)
+    tables = [default, rng.integers(0, 1 << 40, size=256, dtype=np.int64), default,
+              default + rng.integers(0, 2, size=256, dtype=np.int64), rand_i64(rng, (256,), 63)]
+    oracle.set_threads(oracle.max_threads())
+    R = dev(x)
+    t = dev(default.copy())
+    for i, table in enumerate(tables):
+        t.copy_(torch.from_numpy(table))                  # in place: the pointer stays the same
+        expect = getattr(oracle, fn)(x, table)
+        outs = []
+        for rep in range(4):
+            C = torch.empty_like(R)
+            getattr(K.lib, fn)(R.data_ptr(), C.data_ptr(), t.data_ptr(), 1, 1, n)
+            if (rep + i) & 1:
+                torch.cuda.synchronize()
+            outs.append(C)
+        torch.cuda.synchronize()
+        K._check(fn)
+        for rep, C in enumerate(outs):
+            assert np.array_equal(host(C), expect), "table %d, call %d" % (i, rep)
+    oracle.set_threads(1)
+
+
 @pytest.mark.parametrize("T", [1, 7, 64, 100, 1024, 2048, 2050, 3001])
 @pytest.mark.parametrize("with_s2,with_mask,keep_scores", [(True, True, True), (False, False, False), (True, False, True), (False, True, False)])
 def test_softmax_q19_scores_fusion(K, oracle, T, with_s2, with_mask, keep_scores):

@@ -133,17 +133,23 @@ __global__ __launch_bounds__(kActThreads) void act_kernel(const int64_t *__restr
 // values.  A pre-kernel computes them from the caller's table with the same integer arithmetic as act_one;
 // the streaming kernel keeps them in LDS (48-52 KB) and does one 4-byte lookup per element instead of a
 // divide.  Elements outside that range, or a table whose quotients do not fit 32 bits, take act_one.
+//
+// The quotients are kept from call to call (callers pass the same table every time) but never trusted: the
+// pre-kernel leaves a copy of the table it worked from, every workgroup of the streaming kernel compares the
+// caller's table with that copy while it loads it, and on a difference it divides per element like the small
+// kernel and raises a flag in pinned host memory, which makes the next call build the quotients again.
 template <int Q> struct QTab {
     static constexpr int kLo = -(Q + 1), kHi = Q, kRows = kHi - kLo + 1, kEntries = kRows * 256;
 };
 
 template <int Q>
 __global__ __launch_bounds__(256) void act_qtab_kernel(const int64_t *__restrict__ lut, uint32_t *__restrict__ qtab,
-                                                       int *__restrict__ ok)
+                                                       int *__restrict__ ok, int64_t *__restrict__ lut_copy)
 {
     constexpr int64_t ONE = (int64_t)1 << Q;
     const int k = QTab<Q>::kLo + (int)blockIdx.x;
     const int64_t t = lut[threadIdx.x];
+    if (blockIdx.x == 0) lut_copy[threadIdx.x] = t;
     int64_t u;
     if (k < 0) u = t >> (-k);
     else u = (int64_t)((uint64_t)t << k);
@@ -161,14 +167,21 @@ template <int Q, bool SIGMOID, bool GATED>
 __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *__restrict__ R, int64_t *__restrict__ C,
                                                                 const int64_t *__restrict__ lut_g,
                                                                 const uint32_t *__restrict__ qtab_g,
-                                                                const int *__restrict__ ok_g, long n, ActGate gate)
+                                                                const int *__restrict__ ok_g,
+                                                                const int64_t *__restrict__ lut_copy_g, int *stale_host,
+                                                                long n, ActGate gate)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char act_smem[];
     int64_t *lut = reinterpret_cast<int64_t *>(act_smem);
     uint32_t *qtab = reinterpret_cast<uint32_t *>(act_smem + 2048);
     constexpr int64_t LIM = (int64_t)64 << Q;
     constexpr int64_t ONE = (int64_t)1 << Q;
-    if (threadIdx.x < 256) lut[threadIdx.x] = lut_g[threadIdx.x];
+    int differs = 0;                     // the caller's table against the one the quotients were made from
+    if (threadIdx.x < 256) {
+        const int64_t t = lut_g[threadIdx.x];
+        lut[threadIdx.x] = t;
+        differs = t != lut_copy_g[threadIdx.x];
+    }
     for (int i = threadIdx.x; i < QTab<Q>::kEntries / 4; i += kTabThreads)
         reinterpret_cast<v4i_e *>(qtab)[i] = reinterpret_cast<const v4i_e *>(qtab_g)[i];
     __shared__ int ok_s;
@@ -177,8 +190,9 @@ __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *_
         for (int i = 0; i < QTab<Q>::kRows; i++) all &= ok_g[i];
         ok_s = all;
     }
-    __syncthreads();
-    const bool ok = ok_s != 0;
+    const int stale = __syncthreads_or(differs);
+    const bool ok = ok_s != 0 && !stale;
+    if (stale && stale_host && blockIdx.x == 0 && threadIdx.x == 0) *stale_host = 1;
 
     auto one = [&](int64_t r) -> int64_t {
         if (r >= LIM) return r;
@@ -229,9 +243,14 @@ __global__ __launch_bounds__(kTabThreads) void act_table_kernel(const int64_t *_
     }
 }
 
-static uint32_t *g_qtab = nullptr;      // (2Q+2)*256 quotients + the ok flag behind them, kept for the process lifetime
+// Per Q, kept for the process lifetime: (2Q+2)*256 quotients, the ok flags of their rows, the table they were made from.
 constexpr size_t kQtabBytes = (size_t)QTab<25>::kEntries * 4;
 constexpr size_t kQtabFlagBytes = (size_t)QTab<25>::kRows * 4;
+constexpr size_t kQtabLutOffset = (kQtabBytes + kQtabFlagBytes + 15) & ~(size_t)15;
+struct QtabCache { uint32_t *dev = nullptr; bool built = false; };
+static QtabCache g_qtab_cache[2];       // Q23, Q25
+static int *g_qtab_stale = nullptr;     // pinned host memory, one flag per Q: a streaming kernel met another table than the cached one
+static bool g_qtab_stale_tried = false;
 
 template <int Q, bool SIGMOID, bool GATED = false>
 static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim,
@@ -243,13 +262,27 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
     if (!R || !C || !lut || (GATED && !gate.U)) { set_error(kBadArgument, "%s: null pointer", name); return; }
     bool vec = (((uintptr_t)R | (uintptr_t)C | (uintptr_t)gate.U | (uintptr_t)gate.S) & 15) == 0;
     if (vec && n >= (1L << 20)) {
-        if (!g_qtab && hipMalloc(&g_qtab, kQtabBytes + kQtabFlagBytes) != hipSuccess) {
+        QtabCache &qc = g_qtab_cache[Q == 23 ? 0 : 1];
+        if (!qc.dev && hipMalloc(&qc.dev, kQtabLutOffset + 2048) != hipSuccess) {
             (void)hipGetLastError();
-            g_qtab = nullptr;
+            qc.dev = nullptr;
         }
-        if (g_qtab) {
+        if (!g_qtab_stale_tried) {
+            g_qtab_stale_tried = true;
+            if (hipHostMalloc(&g_qtab_stale, 2 * sizeof(int), hipHostMallocDefault) == hipSuccess) g_qtab_stale[0] = g_qtab_stale[1] = 0;
+            else { (void)hipGetLastError(); g_qtab_stale = nullptr; }
+        }
+        if (qc.dev) {
+            uint32_t *g_qtab = qc.dev;
             int *ok = reinterpret_cast<int *>(reinterpret_cast<unsigned char *>(g_qtab) + kQtabBytes);
-            act_qtab_kernel<Q><<<dim3(QTab<Q>::kRows), dim3(256), 0, 0>>>(lut, g_qtab, ok);
+            int64_t *lut_copy = reinterpret_cast<int64_t *>(reinterpret_cast<unsigned char *>(g_qtab) + kQtabLutOffset);
+            // without the pinned flag nothing could report a changed table: the quotients are then made on every call
+            int *stale = g_qtab_stale ? g_qtab_stale + (Q == 23 ? 0 : 1) : nullptr;
+            if (!qc.built || !stale || *reinterpret_cast<volatile int *>(stale)) {
+                if (stale) *reinterpret_cast<volatile int *>(stale) = 0;
+                act_qtab_kernel<Q><<<dim3(QTab<Q>::kRows), dim3(256), 0, 0>>>(lut, g_qtab, ok, lut_copy);
+                qc.built = true;
+            }
             const size_t lds = 2048 + (size_t)QTab<Q>::kEntries * 4;
             static bool raised = false;
             if (!raised) {
@@ -263,7 +296,7 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
             const long per_block = (long)kTabThreads * kActUnroll;
             long blocks = ((n >> 1) + per_block - 1) / per_block;
             if (blocks > 512) blocks = 512;            // persistent (2 per CU): each workgroup loads the table once
-            act_table_kernel<Q, SIGMOID, GATED><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, n, gate);
+            act_table_kernel<Q, SIGMOID, GATED><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, lut_copy, stale, n, gate);
             check_launch(name);
             return;
         }
