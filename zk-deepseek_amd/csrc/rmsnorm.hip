@@ -351,8 +351,8 @@ __global__ __launch_bounds__(kRmsThreads) void rms_apply_kernel(const int64_t *_
 // compute unit, which is what hides the serial stretch (reduction, division, square root) in the middle.
 // VEC: N is even and the rows are 16-byte aligned: elements are moved two at a time with streaming accesses.
 // WPE: waves per SIMD the register allocation must leave room for.  Rows of 4K-8K elements run three workgroups of
-// eight waves per compute unit (WPE 6, 80 registers): measured, a third row in flight is worth more than the few
-// registers spilled for it, a fourth is not.
+// eight waves per compute unit (WPE 6, 80 registers): measured, a third row in flight pays; a fourth (64 registers)
+// spills again and does not.
 // RES: the row that is normalised is A + Y * 2^k (wrapping int64 arithmetic, as the tensor ops of the reference's
 // residual connection, inference/model.py:1465, 1472), and that sum is also stored to Xout (which may be A itself).
 struct RmsResidual { const int64_t *Y; int64_t *Xout; int k; };
@@ -367,7 +367,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
     const long row = blockIdx.x;
     const int64_t *a = A + row * N;
     int64_t v[EPT];
-    WPair<WT> wp[EPT / 2];          // the weights travel with the row: no load is left for after the barrier
+    // The weights travel with the row: no load is left for after the barrier.  Where several rows share a compute unit
+    // through a tight register budget (WPE > 1), int32 weights wait in LDS instead of registers (each thread reads
+    // back only what it wrote itself): the registers they held were being spilled to scratch memory, and those
+    // stores reached HBM (a tenth more bytes written than the output has).
+    constexpr bool W_LDS = VEC && sizeof(WT) == 4 && WPE > 1;
+    __shared__ WPair<WT> w_s[W_LDS ? (EPT / 2) * THREADS : 1];
+    WPair<WT> wp[W_LDS ? 1 : EPT / 2];
     const bool w_vec = ((uintptr_t)W & 7) == 0;
     SquareSum sq;
     if (VEC) {
@@ -376,7 +382,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
             const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
                 const v4i_r t = __builtin_nontemporal_load(reinterpret_cast<const v4i_r *>(a + i));
-                wp[j] = load_w_pair(W, i, w_vec);
+                if (W_LDS) w_s[j * THREADS + threadIdx.x] = load_w_pair(W, i, w_vec);
+                else wp[j] = load_w_pair(W, i, w_vec);
                 v[2 * j] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
                 v[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
                 if (RES) {
@@ -424,8 +431,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
             const int i = (j * THREADS + threadIdx.x) * 2;
             if (i < N) {
                 bool ok0, ok1;
-                const int64_t c0 = rms_apply_quick(v[2 * j], wp[j].x, inv_r, fast_r, ok0);
-                const int64_t c1 = rms_apply_quick(v[2 * j + 1], wp[j].y, inv_r, fast_r, ok1);
+                const WPair<WT> w = W_LDS ? w_s[j * THREADS + threadIdx.x] : wp[W_LDS ? 0 : j];
+                const int64_t c0 = rms_apply_quick(v[2 * j], w.x, inv_r, fast_r, ok0);
+                const int64_t c1 = rms_apply_quick(v[2 * j + 1], w.y, inv_r, fast_r, ok1);
                 redo |= (ok0 ? 0u : 1u << (2 * j)) | (ok1 ? 0u : 2u << (2 * j));
                 const v4i_r t = { (int)(uint32_t)c0, (int)(uint32_t)((uint64_t)c0 >> 32), (int)(uint32_t)c1,
                                   (int)(uint32_t)((uint64_t)c1 >> 32) };
@@ -437,8 +445,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
 #pragma unroll
             for (int j = 0; j < EPT / 2; j++) {
                 const int i = (j * THREADS + threadIdx.x) * 2;
-                if (redo & (1u << (2 * j))) C[row * N + i] = rms_apply_one(v[2 * j], wp[j].x, r, inv_r, fast_r);
-                if (redo & (2u << (2 * j))) C[row * N + i + 1] = rms_apply_one(v[2 * j + 1], wp[j].y, r, inv_r, fast_r);
+                const WPair<WT> w = W_LDS ? w_s[j * THREADS + threadIdx.x] : wp[W_LDS ? 0 : j];
+                if (redo & (1u << (2 * j))) C[row * N + i] = rms_apply_one(v[2 * j], w.x, r, inv_r, fast_r);
+                if (redo & (2u << (2 * j))) C[row * N + i + 1] = rms_apply_one(v[2 * j + 1], w.y, r, inv_r, fast_r);
             }
         }
     } else {
