@@ -394,7 +394,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE))) 
                     v[2 * j + 1] = (int64_t)((uint64_t)v[2 * j + 1] + (y1 << res.k));
                     const v4i_r o = { (int)(uint32_t)v[2 * j], (int)(uint32_t)((uint64_t)v[2 * j] >> 32),
                                       (int)(uint32_t)v[2 * j + 1], (int)(uint32_t)((uint64_t)v[2 * j + 1] >> 32) };
-                    *reinterpret_cast<v4i_r *>(res.Xout + row * N + i) = o;
+                    __builtin_nontemporal_store(o, reinterpret_cast<v4i_r *>(res.Xout + row * N + i));
                 }
                 sq.add(v[2 * j]);
                 sq.add(v[2 * j + 1]);
