@@ -295,7 +295,12 @@ static void launch_act(const char *name, const int64_t *R, int64_t *C, const int
             }
             const long per_block = (long)kTabThreads * kActUnroll;
             long blocks = ((n >> 1) + per_block - 1) / per_block;
-            if (blocks > 512) blocks = 512;            // persistent (2 per CU): each workgroup loads the table once
+            // persistent workgroups, each loads the table once: two per CU; the gate product, with three or four streams
+            // instead of two, runs fastest on 192 workgroups from some tens of millions of elements on (measured on one box
+            // against 128 to 640: [1,8192,18432] 0.608 ms against 0.693 ms on 512, [1,2048,18432] 0.148 against 0.160,
+            // [1,512,18432] 0.039 against 0.038)
+            const long cap = (GATED && n >= (1L << 25)) ? 192 : 512;
+            if (blocks > cap) blocks = cap;
             act_table_kernel<Q, SIGMOID, GATED><<<dim3((unsigned)blocks), dim3(kTabThreads), lds, 0>>>(R, C, lut, g_qtab, ok, lut_copy, stale, n, gate);
             check_launch(name);
             return;
