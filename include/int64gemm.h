@@ -102,6 +102,19 @@ int zk_last_error(void);
 const char *zk_last_error_string(void);
 void zk_clear_error(void);
 
+/* The reference's library allocates nothing and keeps no state; this one keeps scratch buffers on the device between
+ * calls (digit planes of A, partial sums of split tiles, range slots, a row-major copy of a small B, the quotient
+ * tables of the activations), allocated on demand and grown inside a call when a larger problem arrives.
+ * zk_workspace_bytes: device bytes held as scratch right now.  zk_prepared_weights_bytes: device bytes held as digit
+ * planes made by zk_gemm_prepare_weights.  zk_release_workspace: waits for the device and frees the scratch (not the
+ * prepared weights: zk_gemm_release_weights returns those); later calls allocate again what they need. */
+size_t zk_workspace_bytes(void);
+size_t zk_prepared_weights_bytes(void);
+void zk_release_workspace(void);
+/* Reads the diagnosis switches ZK_GEMM_SYNC, ZK_NO_TAIL_SPLIT and ZK_B_ROWS_MIN_MACS from the environment again (they
+ * are read once when the library is loaded, not per call). */
+void zk_reload_env(void);
+
 /* RMS statistic on the device: rms[m] = isqrt((eps + sum_n A[m,n]^2) / dim), exact (192-bit sum).
  * Replaces the host loop of inference/kernel.py:477-494 and :539-542 (one .item() sync per element). */
 void rms_stat_int64(const int64_t *A, int64_t *rms, int M, int N, int64_t eps, int64_t dim);
@@ -169,6 +182,9 @@ long zk_dump_flush(void);
  *   sorted_pos [T*K]: the sorted row of entry (t, k);
  *   tiles [2 * (T*K/32 + E)], ntiles [1]: the 32-row tiles of the segments, for int64_grouped_bmm_launcher;
  *   counts_scratch [E]: scratch.
+ *   An index outside [0, E) belongs to no segment: seg[E] < T*K then, the entry's sorted_pos is 0 (moe_combine reads
+ *   row 0 for it), the unowned rows behind seg[E] get token 0, and the error is recorded once the kernels have run
+ *   (zk_last_error after a synchronisation, or any later call's check); nothing reads outside the buffers.
  * moe_gather_rows: out[r][:] = x[sorted_token[r]][:]  (x [T,N], out [rows,N]).
  * int64_grouped_bmm_launcher: C[r][n] = (sum_k A[r][k] * B_e[n][k]) >> c_rescale (128-bit wrapping sum) and, when R
  *   is not null, R = that sum mod 2^c_rescale, for the rows r of expert e's segment; B_ptrs [groups] holds the
@@ -208,8 +224,11 @@ long zk_gemm_grouped_mfma_calls(void);
  * b_rescale 1 and contiguous rows then read the planes (as many bytes per weight as its values need digits: 3 for
  * |w| < 2^23, 4 up to 31 bits, else 5 or 9) and split nothing of B; results are the same bits.  The library allocates
  * the planes and keeps them until zk_gemm_release_weights or the end of the process.  The original weights must stay
- * where they are and unchanged meanwhile (the exact fallback path and the matrix-vector kernels read them).  Returns 0
- * on success; an error is recorded otherwise.  Waits for the device. */
+ * where they are and unchanged meanwhile (the exact fallback path and the matrix-vector kernels read them).  The planes
+ * are found by ADDRESS and nothing of B is read or range-checked on that path: if the weights are freed without
+ * zk_gemm_release_weights and an allocator hands the address to another matrix of the same shape, that matrix is
+ * multiplied with the old planes and the results are silently wrong.  Release before freeing (the Python wrapper keeps
+ * the tensor alive until release_weights).  Returns 0 on success; an error is recorded otherwise.  Waits for the device. */
 int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K);
 void zk_gemm_release_weights(const void *B);
 /* 1 when the last GEMM-like call ran on the MFMA path and read B from prepared planes, else 0. */

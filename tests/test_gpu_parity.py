@@ -448,15 +448,20 @@ def test_einsum_values_rewritten_with_contiguous_rows(K, oracle, monkeypatch):
     2^32 MACs and more; the threshold is lowered here): ragged T and C, two batches, and a second call with another B
     through the same scratch"""
     monkeypatch.setenv("ZK_B_ROWS_MIN_MACS", "1")
+    K.lib.zk_reload_env()           # the switches are read when the library is loaded, not per call
     rng = np.random.default_rng(77)
     K.lib.zk_gemm_set_path(2)
-    for Bq, S, H, T, Cc in ((2, 9, 5, 70, 45), (1, 40, 3, 33, 130), (1, 3, 16, 257, 64)):
-        for rep in range(2):
-            pr = rng.integers(0, 1 << 19, size=(Bq, S, H, T), dtype=np.int64)
-            kv = rand_i64(rng, (Bq, T, Cc), 36 if rep else 24)
-            assert np.array_equal(host(K.einsum_bsht_btc_bshc(dev(pr), dev(kv), 23)), oracle.einsum_bsht_btc_bshc(pr, kv, 23)), (Bq, S, H, T, Cc, rep)
-            assert K.gemm_last_plan()[0] == 2
-    K.lib.zk_gemm_set_path(0)
+    try:
+        for Bq, S, H, T, Cc in ((2, 9, 5, 70, 45), (1, 40, 3, 33, 130), (1, 3, 16, 257, 64)):
+            for rep in range(2):
+                pr = rng.integers(0, 1 << 19, size=(Bq, S, H, T), dtype=np.int64)
+                kv = rand_i64(rng, (Bq, T, Cc), 36 if rep else 24)
+                assert np.array_equal(host(K.einsum_bsht_btc_bshc(dev(pr), dev(kv), 23)), oracle.einsum_bsht_btc_bshc(pr, kv, 23)), (Bq, S, H, T, Cc, rep)
+                assert K.gemm_last_plan()[0] == 2
+    finally:
+        K.lib.zk_gemm_set_path(0)
+        monkeypatch.delenv("ZK_B_ROWS_MIN_MACS")
+        K.lib.zk_reload_env()
 
 
 def _scores(rng, shape, Q, masked=True):
@@ -960,6 +965,38 @@ def test_moe_dispatch(K, oracle, T, E, Kr):
     tiles = host(d["tiles"])[: 2 * nt].reshape(nt, 2)
     want = [(e, r) for e in range(E) for r in range(int(seg[e]), int(seg[e + 1]), 32)]
     assert tiles.tolist() == [list(t) for t in want]
+
+
+def test_moe_dispatch_reports_indices_outside_the_experts(K, oracle):
+    """an expert index outside [0, E) belongs to no segment: nothing may read outside the buffers (the entry points at
+    row 0, the unowned rows get token 0), the valid entries are placed as ever, and the error channel reports the call"""
+    rng = np.random.default_rng(5)
+    T, E, Kr, N = 50, 16, 4, 64
+    idx = _routing(rng, T, E, Kr)
+    bad = [(3, 1, -1), (20, 0, E), (49, 3, 1 << 40)]
+    for t, k, v in bad:
+        idx[t, k] = v
+    d = K.moe_dispatch(dev(idx), E)
+    torch.cuda.synchronize()
+    assert K.lib.zk_last_error() == 1 and b"outside" in K.lib.zk_last_error_string()
+    K.lib.zk_clear_error()
+    valid = (idx >= 0) & (idx < E)
+    seg, tok, pos = oracle.moe_dispatch(np.where(valid, idx, E), E + 1)      # the invalid ones sorted behind everything else
+    rows = T * Kr - len(bad)
+    assert np.array_equal(host(d["seg"]), seg[: E + 1]) and int(seg[E]) == rows
+    assert np.array_equal(host(d["token"])[:rows], tok[:rows]) and not host(d["token"])[rows:].any()
+    assert np.array_equal(host(d["pos"])[valid], pos[valid]) and not host(d["pos"])[~valid].any()
+    # the steps behind it run on what the dispatch left, inside their buffers
+    x = rand_i64(rng, (T, N), 30)
+    xs = K.moe_gather_rows(dev(x), d)
+    assert np.array_equal(host(xs)[:rows], x[tok[:rows]]) and np.array_equal(host(xs)[rows:], np.broadcast_to(x[0], (len(bad), N)))
+    w = rand_i64(rng, (T, Kr), 23)
+    y = K.moe_combine(xs, dev(w), d, T)
+    p = np.where(valid, pos, 0)
+    ye = np.zeros((T, N), dtype=np.int64)
+    for k in range(Kr):
+        ye += (host(xs)[p[:, k]] * w[:, k:k + 1]) >> 23
+    assert np.array_equal(host(y), ye)
 
 
 @pytest.mark.parametrize("path", PATHS)

@@ -15,6 +15,18 @@ void set_error(int code, const char *fmt, ...);
 // hipGetLastError() after a launch; records kLaunchFailure and returns false on failure.
 bool check_launch(const char *what);
 
+// Errors detected on the device: a pinned host flag per kind (null when pinned memory is not to be had) that a kernel
+// sets to 1; zk_last_error() turns a set flag into a recorded error.
+enum DeferredError { kDeferredMoeIndex = 0, kDeferredCount };
+int *deferred_error_flag(int which);
+
+// Device memory the library holds between calls (per module), and its release.
+size_t gemm_mfma_workspace_bytes(size_t *prepared_bytes);
+void gemm_mfma_release_workspace();
+void gemm_mfma_reload_switches();
+size_t act_workspace_bytes();
+void act_release_workspace();
+
 constexpr int kWave = 64;
 
 // ---- wave-level helpers --------------------------------------------------------------------

@@ -252,6 +252,23 @@ static QtabCache g_qtab_cache[2];       // Q23, Q25
 static int *g_qtab_stale = nullptr;     // pinned host memory, one flag per Q: a streaming kernel met another table than the cached one
 static bool g_qtab_stale_tried = false;
 
+// Device memory held for the quotient tables, and its return (the tables are made again when next needed).
+size_t act_workspace_bytes()
+{
+    size_t n = 0;
+    for (const QtabCache &qc : g_qtab_cache) n += qc.dev ? kQtabLutOffset + 2048 : 0;
+    return n;
+}
+
+void act_release_workspace()
+{
+    for (QtabCache &qc : g_qtab_cache) {
+        if (qc.dev) (void)hipFree(qc.dev);
+        qc.dev = nullptr;
+        qc.built = false;
+    }
+}
+
 template <int Q, bool SIGMOID, bool GATED = false>
 static void launch_act(const char *name, const int64_t *R, int64_t *C, const int64_t *lut, int Bsz, int S, int Dim,
                        ActGate gate = ActGate{ nullptr, nullptr })

@@ -34,9 +34,10 @@ void gemm_valu_launch(const GemmDesc &d, const unsigned long long *guard = nullp
 // guessed.  Returns false (nothing launched) for any other descriptor.
 bool gemm_gemv_launch(const GemmDesc &d);
 
-// Limb-decomposed i8 MFMA.  Returns false (nothing launched) when the descriptor is outside what it
-// supports, in which case the caller falls back to the VALU path.
-bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
+// Limb-decomposed i8 MFMA.  Returns 0 when the product was launched, 1 when the descriptor is outside what it
+// supports or memory for its buffers is short (nothing was launched; the caller falls back to the VALU path), -1 on an
+// error (recorded).  The outcome describes this call only, whatever the sticky error channel holds from earlier ones.
+int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 
 // Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
 // vector-ALU recomputation (known once their range has reached the host).
@@ -80,7 +81,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b);
 // operands wider than its kernels take), group by group through gemm_dispatch after one read-back of the segments.
 void gemm_grouped_dispatch(const char *name, const GroupedDesc &d);
 
-// Top-level dispatch used by the extern "C" launchers.
-void gemm_dispatch(const char *name, const GemmDesc &d);
+// Top-level dispatch used by the extern "C" launchers.  False when this call failed (the error is recorded).
+bool gemm_dispatch(const char *name, const GemmDesc &d);
 
 }  // namespace zk

@@ -11,7 +11,7 @@ static int g_gemm_path = kPathAuto;
 static int g_last_path = 0, g_last_la = 0, g_last_lb = 0;
 static long g_grouped_mfma_calls = 0;
 
-void gemm_dispatch(const char *name, const GemmDesc &d)
+bool gemm_dispatch(const char *name, const GemmDesc &d)
 {
     // one or two rows (a decoding step, the head): the exact vector-ALU stream over the weights, unless the MFMA
     // path is asked for by name
@@ -21,26 +21,26 @@ void gemm_dispatch(const char *name, const GemmDesc &d)
     const bool prepared = g_gemm_path != kPathValu && !d.b32 && (long)d.N * d.K >= (16L << 20) && gemm_mfma_is_prepared(d.B);
     if (g_gemm_path != kPathMfma && !prepared && gemm_gemv_launch(d)) {
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
-        check_launch(name);
-        return;
+        return check_launch(name);
     }
     if (g_gemm_path != kPathValu) {
         int la = 0, lb = 0;
-        if (gemm_mfma_launch(d, &la, &lb)) {
+        // 0: launched, 1: declined (whatever the error channel holds comes from an earlier call and must not keep this
+        // one from running on the other path), -1: failed and recorded
+        const int rc = gemm_mfma_launch(d, &la, &lb);
+        if (rc == 0) {
             g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb;
-            check_launch(name);
-            return;
+            return check_launch(name);
         }
-        if (zk_last_error() != kOk) return;
+        if (rc < 0) return false;
     }
     if (g_gemm_path != kPathMfma && prepared && gemm_gemv_launch(d)) {
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
-        check_launch(name);
-        return;
+        return check_launch(name);
     }
     gemm_valu_launch(d);
     g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
-    check_launch(name);
+    return check_launch(name);
 }
 
 // rows up to which the grouped product is offered to the matrix-vector kernels, which go row by row (a few tokens at
@@ -93,8 +93,7 @@ void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
         g.C = d.C + (long)r0 * d.ldc; g.R = d.R ? d.R + (long)r0 * d.ldc : nullptr; g.ldc = d.ldc; g.sC = 0;
         g.G = 1; g.M = m; g.N = d.N; g.K = d.K;
         g.shift = d.shift; g.init = d.init; g.a_rs = 1; g.b_rs = 1;
-        gemm_dispatch(name, g);
-        if (zk_last_error() != kOk) return;
+        if (!gemm_dispatch(name, g)) return;
     }
 }
 

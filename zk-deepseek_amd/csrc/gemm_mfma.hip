@@ -132,17 +132,39 @@ struct RangeCache {
 
 static RangeCache g_cache;
 
-// Grows a device buffer kept for the process lifetime.  Returns false (buffer left empty) when memory is short.
-template <typename T>
-static bool grow(T *&buf, size_t &have, size_t need, const char *what)
+// Diagnosis switches, read from the environment once when the library is loaded (and again on zk_reload_env):
+// ZK_GEMM_SYNC: every call waits for its own digit verdict; ZK_NO_TAIL_SPLIT: no split-K; ZK_B_ROWS_MIN_MACS: product
+// size from which a small n-contiguous int64 B is rewritten with contiguous rows first.
+struct Switches { bool sync_verdict, no_tail_split; double b_rows_min_macs; };
+constexpr long kBRowsMinMacs = 1L << 32;
+static Switches read_switches()
 {
-    if (need <= have) return true;
-    if (buf && hipFree(buf) != hipSuccess) { set_error(kLaunchFailure, "gemm: cannot release the %s", what); return false; }
+    Switches s;
+    s.sync_verdict = getenv("ZK_GEMM_SYNC") != nullptr;
+    s.no_tail_split = getenv("ZK_NO_TAIL_SPLIT") != nullptr;
+    const char *m = getenv("ZK_B_ROWS_MIN_MACS");
+    s.b_rows_min_macs = m ? atof(m) : (double)kBRowsMinMacs;
+    return s;
+}
+static Switches g_switches = read_switches();
+void gemm_mfma_reload_switches() { g_switches = read_switches(); }
+
+// Outcome of a launcher, derived from the call itself (never from the sticky error channel, which may still hold an
+// error of an earlier, unrelated call): done, declined (nothing launched that the caller may not overwrite: it takes
+// another route) or failed (an error was recorded).
+enum Outcome { kDone = 0, kDeclined = 1, kFailed = -1 };
+
+// Grows a device buffer kept until gemm_mfma_release_workspace.  kDeclined (buffer left empty) when memory is short.
+template <typename T>
+static Outcome grow(T *&buf, size_t &have, size_t need, const char *what)
+{
+    if (need <= have) return kDone;
+    if (buf && hipFree(buf) != hipSuccess) { set_error(kLaunchFailure, "gemm: cannot release the %s", what); return kFailed; }
     buf = nullptr;
     have = 0;
-    if (hipMalloc(&buf, need * sizeof(T)) != hipSuccess) { (void)hipGetLastError(); buf = nullptr; return false; }
+    if (hipMalloc(&buf, need * sizeof(T)) != hipSuccess) { (void)hipGetLastError(); buf = nullptr; return kDeclined; }
     have = need;
-    return true;
+    return kDone;
 }
 
 static bool read_range(unsigned long long *dev, int64_t (&out)[4])
@@ -342,7 +364,11 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
     // the pre-pass that splits A in fragment order does the same for the rows of a weight matrix (64 rows per workgroup)
     const int rows_per_wg = 256 / (4 * pb.kk);
     const dim3 grid((unsigned)(pb.ksteps / pb.kk), (unsigned)((pb.nsub * 32 + rows_per_wg - 1) / rows_per_wg), 1);
-    if (!grow(g_cache.mm, g_cache.mm_count, (size_t)grid.x * grid.y * 2, "range scratch")) { release_prepared(pb); return 1; }
+    if (grow(g_cache.mm, g_cache.mm_count, (size_t)grid.x * grid.y * 2, "range scratch") != kDone) {
+        release_prepared(pb);
+        set_error(kLaunchFailure, "%s: cannot allocate the range scratch", name);
+        return 1;
+    }
     MfmaParams q = {};
     q.lda = K; q.sA = 0; q.M = N; q.K = K;
     for (int i = 0; i < count; i++) {
@@ -370,6 +396,42 @@ int gemm_mfma_prepare(const void *B, int b32, int groups, int N, int K)
     return 0;
 }
 
+// Device memory the GEMM path holds right now: its scratch buffers, and the digit planes of prepared weights.
+size_t gemm_mfma_workspace_bytes(size_t *prepared_bytes)
+{
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    size_t scratch = g_cache.dev ? (8 + 4 * kFoldParts) * sizeof(unsigned long long) : 0;
+    scratch += g_cache.planes_bytes + (g_cache.mm_count + g_cache.wg_count + g_cache.partials_bytes) * sizeof(unsigned long long) +
+               g_cache.b_rows_count * sizeof(int64_t);
+    size_t prepared = 0;
+    for (const auto &kv : g_prepared) {
+        const PreparedB &pb = kv.second;
+        const size_t count = pb.groups > 0 ? (size_t)pb.groups : 1;
+        prepared += (size_t)pb.nsub * pb.ksteps * pb.nb * 1024 * count + (pb.table ? count * sizeof(void *) : 0);
+    }
+    if (prepared_bytes) *prepared_bytes = prepared;
+    return scratch;
+}
+
+// Gives the scratch buffers back (they grow again on demand).  Waits for the device first: launches that use them may
+// still be under way.  Prepared weights stay (zk_gemm_release_weights returns those).
+void gemm_mfma_release_workspace()
+{
+    std::lock_guard<std::mutex> lock(g_cache.mu);
+    (void)hipDeviceSynchronize();
+    drain_pending();
+    if (g_cache.planes) (void)hipFree(g_cache.planes);
+    if (g_cache.mm) (void)hipFree(g_cache.mm);
+    if (g_cache.wg) (void)hipFree(g_cache.wg);
+    if (g_cache.partials) (void)hipFree(g_cache.partials);
+    if (g_cache.b_rows) (void)hipFree(g_cache.b_rows);
+    g_cache.planes = nullptr; g_cache.planes_bytes = 0;
+    g_cache.mm = nullptr; g_cache.mm_count = 0;
+    g_cache.wg = nullptr; g_cache.wg_count = 0;
+    g_cache.partials = nullptr; g_cache.partials_bytes = 0;
+    g_cache.b_rows = nullptr; g_cache.b_rows_count = 0;
+}
+
 // B[g][k][n] (n contiguous) -> out[g][n][k]: 32x32 tiles through LDS, both sides coalesced
 __global__ __launch_bounds__(256) void b_rows_kernel(const int64_t *__restrict__ B, long ldbk, long sB, int64_t *__restrict__ out, int N, int K)
 {
@@ -395,23 +457,22 @@ __global__ __launch_bounds__(256) void b_rows_kernel(const int64_t *__restrict__
 // probabilities, `bsht,btc->bshc`) is worth rewriting with contiguous rows first: the row-major kernels read it with
 // 16-byte loads and take A from digit planes (measured at S = T = 1024, 128 heads: 1.67 -> 1.45 ms, the rewrite 9 us).
 constexpr long kBRowsMaxElements = 8L << 20;         // 64 MB
-constexpr long kBRowsMinMacs = 1L << 32;
 
-bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
+int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
 {
     // Operand divisors: a power of two on B is folded into the digit split of the 32-row kernels (the head projection
     // divides its weights by 256, inference/model.py:1519, and runs on the last token only); anything else: VALU path.
     int b_shift = 0;
-    if (d.a_rs != 1) return false;
+    if (d.a_rs != 1) return kDeclined;
     if (d.b_rs != 1) {
-        if (d.b_rs <= 0 || (d.b_rs & (d.b_rs - 1)) != 0 || d.M > 32) return false;
+        if (d.b_rs <= 0 || (d.b_rs & (d.b_rs - 1)) != 0 || d.M > 32) return kDeclined;
         while (((int64_t)1 << b_shift) < d.b_rs) b_shift++;
     }
-    if (d.K <= 0 || d.M <= 0 || d.N <= 0 || d.G <= 0) return false;
-    if (d.G > 65535) return false;
+    if (d.K <= 0 || d.M <= 0 || d.N <= 0 || d.G <= 0) return kDeclined;
+    if (d.G > 65535) return kDeclined;
     bool kmajor = d.ldbn == 1 && d.ldbk != 1;
     std::lock_guard<std::mutex> lock(g_cache.mu);
-    if (!init_cache()) return false;
+    if (!init_cache()) return kFailed;
     drain_pending();
 
     MfmaParams p = {};
@@ -427,15 +488,16 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     }
     const long b_batches = d.sB != 0 ? d.G : 1;
     if (kmajor && !d.b32 && d.M > 32 && b_batches * d.N * d.K <= kBRowsMaxElements &&
-        (double)d.G * d.M * d.N * d.K >= (getenv("ZK_B_ROWS_MIN_MACS") ? atof(getenv("ZK_B_ROWS_MIN_MACS")) : (double)kBRowsMinMacs)) {
+        (double)d.G * d.M * d.N * d.K >= g_switches.b_rows_min_macs) {
         // (without memory for the copy the n-contiguous kernels run as before)
-        if (grow(g_cache.b_rows, g_cache.b_rows_count, (size_t)(b_batches * d.N * d.K), "row-major copy of B")) {
+        const Outcome got = grow(g_cache.b_rows, g_cache.b_rows_count, (size_t)(b_batches * d.N * d.K), "row-major copy of B");
+        if (got == kDone) {
             const dim3 grid((unsigned)((d.N + 31) / 32), (unsigned)((d.K + 31) / 32), (unsigned)b_batches);
             b_rows_kernel<<<grid, dim3(256), 0, 0>>>(reinterpret_cast<const int64_t *>(d.B), d.ldbk, d.sB, g_cache.b_rows, d.N, d.K);
             p.B = g_cache.b_rows; p.ldbn = d.K; p.ldbk = 1; p.sB = d.sB != 0 ? (long)d.N * d.K : 0;
             kmajor = false;
-        } else if (zk_last_error() != kOk) {
-            return false;
+        } else if (got == kFailed) {
+            return kFailed;
         }
     }
     p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift; p.init = d.init;
@@ -454,7 +516,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
     }
     // Operands seen before: speculate, do not wait.  Otherwise sample them and check the verdict before returning.
     PendingRange *slot = nullptr;
-    if (na && nb && g_cache.pinned && getenv("ZK_GEMM_SYNC") == nullptr) {
+    if (na && nb && g_cache.pinned && !g_switches.sync_verdict) {
         PendingRange &s = g_cache.pending[g_cache.pending_head];
         if (!s.busy && s.ev) slot = &s;
     }
@@ -464,7 +526,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         range_sample_kernel<<<1, 256, 0, 0>>>(p, d.b32, d.G, 0);
         range_sample_kernel<<<1, 256, 0, 0>>>(p, d.b32, d.G, 1);
         int64_t r[4];
-        if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
+        if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return kFailed; }
         if (!na) na = limbs_needed(r[0], r[1]);
         if (!nb) nb = limbs_needed(r[2], r[3]);
     }
@@ -484,11 +546,11 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
             if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag);
         }
-        if (!inst) return false;
+        if (!inst) return kDeclined;
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
         const int ksteps = ((d.K + 32 * inst->kk - 1) / (32 * inst->kk)) * inst->kk;     // 32-k steps, padded
-        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return false;
+        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return kDeclined;
         const int BM = inst->bm, BN = inst->bn;
         p.tiles_m = (d.M + BM - 1) / BM;
         p.tiles_n = (d.N + BN - 1) / BN;
@@ -497,19 +559,19 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         const size_t b_bytes = (size_t)d.N * d.K * (d.b32 ? 4 : 8);
         p.n_fastest = (b_bytes <= ((size_t)8 << 20) && p.tiles_n > 1 && p.tiles_m > 1) ? 1 : 0;
         const long per_batch = (long)p.tiles_m * p.tiles_n;
-        if (per_batch > 0x7FFFFFFFL) return false;
+        if (per_batch > 0x7FFFFFFFL) return kDeclined;
         const long total = per_batch * d.G;
-        if (total > 0x7FFFFFFFL / 8) return false;
+        if (total > 0x7FFFFFFFL / 8) return kDeclined;
         // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass (never for the
         // 32-row tiles: splitting a handful of rows on the fly is cheaper than another kernel in front)
         const bool use_planes = !kmajor && (p.tiles_n >= 4 || prep) && !inst->skinny;
-        if (b_shift && (kmajor || !inst->skinny)) return false;
+        if (b_shift && (kmajor || !inst->skinny)) return kDeclined;
         const int variant = prep ? (inst->skinny ? kB64FlyBPlanes : kB64PlanesBoth)
                           : b_shift ? (d.b32 ? kB32FlyRs : kB64FlyRs)
                           : kmajor ? (d.b32 ? kB32KmajorFly : kB64KmajorFly)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
-        if (!fn) return false;
+        if (!fn) return kDeclined;
 
         // Split-K: a launch smaller than the device is cut into `split` slices of K per tile, each a workgroup of
         // its own; with more tiles than compute units the same is done for the tiles of the last, partial round
@@ -522,7 +584,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         p.partials = nullptr;
         p.part64 = 0;
         p.finish_rq = 4;
-        if (getenv("ZK_NO_TAIL_SPLIT") == nullptr) {
+        if (!g_switches.no_tail_split) {
             if (total < g_cache.cus) {
                 tail = (int)total;
                 split = g_cache.cus / tail;
@@ -549,17 +611,18 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             while ((1L << kbits) < (long)ksteps * 32) kbits++;
             const bool part64 = 8 * (inst->na + inst->nb) - 2 + kbits <= 62;
             const size_t need = (size_t)tail * split * BM * BN * (part64 ? 1 : 2);
-            if (grow(g_cache.partials, g_cache.partials_bytes, need, "partial-sum buffer")) {
+            const Outcome got = grow(g_cache.partials, g_cache.partials_bytes, need, "partial-sum buffer");
+            if (got == kDone) {
                 p.main_tiles = (int)(total - tail);
                 p.split = split;
                 p.tail_xcd = (!p.n_fastest && d.G == 1 && tail % p.tiles_m == 0 && p.main_tiles % 8 == 0 &&
                               ((long)tail * split) % (8L * p.tiles_m) == 0) ? 1 : 0;
                 p.partials = g_cache.partials;
                 p.part64 = part64 ? 1 : 0;
-            } else if (zk_last_error() != kOk) return false;
+            } else if (got == kFailed) return kFailed;
         }
         const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
-        if (!grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return false;
+        if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;
         p.wg_range = g_cache.wg;
 
         long plane_wgs = 0;
@@ -568,12 +631,12 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             const int msub = p.tiles_m * (BM / 32);
             const size_t need = (size_t)d.G * msub * ksteps * inst->na * 1024;
             // not enough memory for planes: the caller uses the VALU path
-            if (!grow(g_cache.planes, g_cache.planes_bytes, need, "digit-plane buffer")) return false;
+            if (const Outcome got = grow(g_cache.planes, g_cache.planes_bytes, need, "digit-plane buffer")) return got;
             p.a_planes = g_cache.planes; p.a_msub = msub; p.a_ksteps = ksteps;
             const int rows_per_wg = 256 / (4 * inst->kk);
             const dim3 pgrid((unsigned)(ksteps / inst->kk), (unsigned)((msub * 32 + rows_per_wg - 1) / rows_per_wg), (unsigned)d.G);
             plane_wgs = (long)pgrid.x * pgrid.y * pgrid.z;
-            if (!grow(g_cache.mm, g_cache.mm_count, (size_t)plane_wgs * 2, "range scratch")) return false;
+            if (const Outcome got = grow(g_cache.mm, g_cache.mm_count, (size_t)plane_wgs * 2, "range scratch")) return got;
             // (the owned-k pattern of the planes of A follows the kernel that reads them: prepared planes of B go with the int64 forms)
             inst->planes[(d.b32 && !prep) ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
         }
@@ -582,7 +645,7 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
             if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
                 set_error(kLaunchFailure, "gemm: cannot raise the LDS limit to %zu bytes", lds);
-                return false;
+                return kFailed;
             }
             lds_raised.insert((const void *)fn);
         }
@@ -594,13 +657,13 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             if (err != hipSuccess) {
                 set_error(kLaunchFailure, "gemm: MFMA kernel launch failed (%s; digits %d,%d, %ld workgroups of %d threads, %zu bytes of LDS)",
                           hipGetErrorString(err), inst->na, inst->nb, blocks, inst->threads, lds);
-                return false;
+                return kFailed;
             }
         }
         const FoldArgs fold = make_fold(g_cache.mm, plane_wgs, g_cache.wg, blocks, p.range, inst->na, inst->nb, slot ? slot->host : nullptr);
         if (p.split > 1) {
             inst->finish<<<dim3((unsigned)((total - p.main_tiles) * p.finish_rq + fold.parts)), dim3((unsigned)inst->threads), 0, 0>>>(p, fold);
-            if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return false; }
+            if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: split finish launch failed"); return kFailed; }
         } else {
             range_fold_kernel<<<dim3((unsigned)fold.parts), 256, 0, 0>>>(fold);
         }
@@ -617,18 +680,18 @@ bool gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             } else {
                 (void)hipGetLastError();
             }
-            return true;
+            return kDone;
         }
         int64_t r[4];
-        if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return false; }
+        if (!read_range(p.range, r)) { set_error(kLaunchFailure, "gemm: range readback failed"); return kFailed; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = prep ? prep->nb : limbs_needed(r[2], r[3]);
         g_cache.store_pair(key_a, need_a, key_b, need_b);
-        if (need_a <= inst->na && need_b <= inst->nb) return true;
+        if (need_a <= inst->na && need_b <= inst->nb) return kDone;
         na = need_a;
         nb = need_b;
     }
     set_error(kLaunchFailure, "gemm: digit count did not settle");
-    return false;
+    return kFailed;
 }
 
 int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
@@ -690,7 +753,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         const long blocks = max_mtiles * p.tiles_n;
         if (blocks > 0x7FFFFFFFL / 8) return 1;
         p.main_tiles = (int)blocks;
-        if (!grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return zk_last_error() != kOk ? -1 : 1;
+        if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;
         p.wg_range = g_cache.wg;
         const size_t lds = 2 * (size_t)inst->kk * ((inst->bm / 32) * inst->na + (inst->bn / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
         static std::set<const void *> lds_raised;

@@ -29,8 +29,12 @@ __global__ __launch_bounds__(256) void moe_count_kernel(const int64_t *__restric
 
 // exclusive scan of the counts and the table of 32-row tiles: one workgroup, 256 experts per round (a single thread
 // walking 256 counts took 19 us, longer than every other step of a one-token dispatch)
+// Entries whose expert index lies outside [0, E) are counted by no workgroup: the rows behind the last segment then
+// belong to nobody.  Their tokens are set to 0 here (so that a gather reads valid memory) and `bad_host`, a flag in
+// pinned host memory, reports the call.
 __global__ __launch_bounds__(256) void moe_scan_kernel(const int *__restrict__ counts, int E, int *__restrict__ seg, int *__restrict__ tiles,
-                                                       int *__restrict__ ntiles)
+                                                       int *__restrict__ ntiles, long entries, int *__restrict__ sorted_token,
+                                                       int *bad_host)
 {
     __shared__ int wave_sum[2][4];
     __shared__ int carry[2];                       // rows and tiles of the rounds before this one
@@ -59,7 +63,10 @@ __global__ __launch_bounds__(256) void moe_scan_kernel(const int *__restrict__ c
         if (threadIdx.x == 255) { carry[0] = bc + pc; carry[1] = bt + pt; }
         __syncthreads();
     }
-    if (threadIdx.x == 0) { seg[E] = carry[0]; ntiles[0] = carry[1]; }
+    const int placed = carry[0];
+    if (threadIdx.x == 0) { seg[E] = placed; ntiles[0] = carry[1]; }
+    for (long r = placed + (long)threadIdx.x; r < entries; r += 256) sorted_token[r] = 0;
+    if (threadIdx.x == 0 && placed != entries && bad_host) *bad_host = 1;
 }
 
 // workgroup e walks the entries in order and gives its own consecutive rows: a stable partition
@@ -74,7 +81,10 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int64_t *__restric
     __syncthreads();
     for (long start = 0; start < entries; start += 256) {
         const long i = start + threadIdx.x;
-        const bool mine = i < entries && indices[i] == e;
+        const int64_t idx = i < entries ? indices[i] : -1;
+        const bool mine = i < entries && idx == e;
+        // an index outside [0, E) belongs to no workgroup: its entry points at row 0 rather than at whatever the buffer held
+        if (e == 0 && i < entries && (idx < 0 || idx >= (int64_t)gridDim.x)) sorted_pos[i] = 0;
         const unsigned long long ballot = __ballot(mine);
         const int before = __popcll(ballot & ((1ull << lane) - 1));
         if (lane == 0) wave_count[wave] = __popcll(ballot);
@@ -141,7 +151,8 @@ void moe_dispatch(const int64_t *indices, int T, int K, int E, int *counts_scrat
     if (E > 65535) { zk::set_error(zk::kUnsupportedSize, "%s: more than 65535 experts", name); return; }
     const long entries = (long)T * K;
     zk::moe_count_kernel<<<dim3((unsigned)E), dim3(256), 0, 0>>>(indices, entries, counts_scratch);
-    zk::moe_scan_kernel<<<dim3(1), dim3(256), 0, 0>>>(counts_scratch, E, seg, tiles, ntiles);
+    zk::moe_scan_kernel<<<dim3(1), dim3(256), 0, 0>>>(counts_scratch, E, seg, tiles, ntiles, entries, sorted_token,
+                                                      zk::deferred_error_flag(zk::kDeferredMoeIndex));
     if (entries > 0) zk::moe_place_kernel<<<dim3((unsigned)E), dim3(256), 0, 0>>>(indices, entries, K, seg, sorted_token, sorted_pos);
     zk::check_launch(name);
 }

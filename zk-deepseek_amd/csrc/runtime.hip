@@ -25,6 +25,38 @@ void set_error(int code, const char *fmt, ...)
     if (getenv("ZK_VERBOSE")) fprintf(stderr, "libint64gemm: %s\n", g_err_text);
 }
 
+// Errors that only a kernel can detect travel through pinned host memory: the kernel stores 1 into its flag, and the
+// next look at the error channel after that store has landed records the error.
+static int *g_deferred = nullptr;
+static bool g_deferred_tried = false;
+static const char *const kDeferredText[kDeferredCount] = {
+    "moe_dispatch: an expert index lies outside [0, E); its entries were left out (they read row 0 in moe_combine)",
+};
+
+int *deferred_error_flag(int which)
+{
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    if (!g_deferred_tried) {
+        g_deferred_tried = true;
+        if (hipHostMalloc(&g_deferred, kDeferredCount * sizeof(int), hipHostMallocDefault) == hipSuccess) {
+            for (int i = 0; i < kDeferredCount; i++) g_deferred[i] = 0;
+        } else {
+            (void)hipGetLastError();
+            g_deferred = nullptr;
+        }
+    }
+    return g_deferred ? g_deferred + which : nullptr;
+}
+
+static void take_deferred_errors()
+{
+    if (!g_deferred) return;
+    for (int i = 0; i < kDeferredCount; i++) {
+        volatile int *f = g_deferred + i;
+        if (*f) { *f = 0; set_error(kBadArgument, "%s", kDeferredText[i]); }
+    }
+}
+
 bool check_launch(const char *what)
 {
     hipError_t e = hipGetLastError();
@@ -41,6 +73,7 @@ extern "C" {
 
 int zk_last_error(void)
 {
+    zk::take_deferred_errors();
     std::lock_guard<std::mutex> lock(zk::g_err_mutex);
     return zk::g_err_code;
 }
@@ -53,6 +86,26 @@ void zk_clear_error(void)
     zk::g_err_code = zk::kOk;
     zk::g_err_text[0] = 0;
 }
+
+size_t zk_workspace_bytes(void)
+{
+    return zk::gemm_mfma_workspace_bytes(nullptr) + zk::act_workspace_bytes();
+}
+
+size_t zk_prepared_weights_bytes(void)
+{
+    size_t prepared = 0;
+    (void)zk::gemm_mfma_workspace_bytes(&prepared);
+    return prepared;
+}
+
+void zk_release_workspace(void)
+{
+    zk::gemm_mfma_release_workspace();       // waits for the device first
+    zk::act_release_workspace();
+}
+
+void zk_reload_env(void) { zk::gemm_mfma_reload_switches(); }
 
 void zk_timer_start(void)
 {

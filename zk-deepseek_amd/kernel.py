@@ -87,6 +87,8 @@ lib.zk_dump_host.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
 lib.zk_dump_flush.restype = ctypes.c_long
 lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
+lib.zk_workspace_bytes.restype = ctypes.c_size_t
+lib.zk_prepared_weights_bytes.restype = ctypes.c_size_t
 
 
 def _check(what):
@@ -97,11 +99,18 @@ def _check(what):
         raise RuntimeError("%s failed (code %d): %s" % (what, code, msg))
 
 
-def prepare_weights(W, groups=0, N=None, K=None, b32=False):
+# Prepared planes are found by the address of the weights, and nothing of B is read or checked on that path: were the
+# tensor freed, torch's allocator could hand its address to another weight matrix of the same shape, which would then be
+# multiplied with the old planes.  So the tensors (for a pointer table: the table and, when given, the matrices it points
+# at) are kept alive here until release_weights.
+_prepared_keepalive = {}
+
+
+def prepare_weights(W, groups=0, N=None, K=None, b32=False, matrices=None):
     """Split a weight matrix [N,K] (int64 or int32) or, with groups > 0, every matrix of the device pointer table `W` made
-    by pointer_table (b32 says whether they are int32) into digit planes once; later int64_bmm_broadcast /
-    int64_grouped_bmm calls with the same tensor read the planes instead of splitting the weights in every tile.  The
-    weights must not change until release_weights."""
+    by pointer_table (b32 says whether they are int32; pass the tensors themselves as `matrices` so that they are kept
+    alive too) into digit planes once; later int64_bmm_broadcast / int64_grouped_bmm calls with the same tensor read the
+    planes instead of splitting the weights in every tile.  The weights must not change until release_weights."""
     assert W.is_cuda and W.is_contiguous()
     if groups == 0:
         assert W.dim() == 2 and W.dtype in (torch.int64, torch.int32)
@@ -111,10 +120,22 @@ def prepare_weights(W, groups=0, N=None, K=None, b32=False):
         assert W.dtype == torch.int64 and W.numel() == groups
     if lib.zk_gemm_prepare_weights(W.data_ptr(), 1 if b32 else 0, int(groups), int(N), int(K)) != 0:
         _check("prepare_weights")
+    _prepared_keepalive[W.data_ptr()] = (W, matrices)
 
 
 def release_weights(W):
     lib.zk_gemm_release_weights(W.data_ptr())
+    _prepared_keepalive.pop(W.data_ptr(), None)
+
+
+def workspace_bytes():
+    """(scratch bytes, bytes of prepared digit planes) the library holds on the device right now"""
+    return int(lib.zk_workspace_bytes()), int(lib.zk_prepared_weights_bytes())
+
+
+def release_workspace():
+    """waits for the device and frees the library's scratch buffers (they are allocated again on demand)"""
+    lib.zk_release_workspace()
 
 
 def gemm_last_pairs():
@@ -243,8 +264,11 @@ rms = torch.zeros((500,), dtype=torch.int64, device="cpu")
 rms_gpu = None
 
 
-def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim):
-    """C = floor(A * W / rms) per row, rms = isqrt((eps + sum a^2) // dim).  Returns (C, rms buffer)."""
+def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim, host_rms=True):
+    """C = floor(A * W / rms) per row, rms = isqrt((eps + sum a^2) // dim).  Returns (C, rms buffer): the 500-row host
+    buffer of the reference (inference/kernel.py:525, 550).  host_rms=False (not in the reference) returns the 500-row
+    DEVICE buffer instead and does not wait for the GPU: a caller that only dumps the statistic (saveTensor takes device
+    tensors) keeps the layer asynchronous."""
     global rms, rms_gpu
     assert A.dtype == torch.int64
     assert A.is_cuda and W.is_cuda
@@ -260,11 +284,13 @@ def RMS_Norm_int64(A: torch.Tensor, W: torch.Tensor, eps, dim):
         assert W.dtype == torch.int64
         lib.rms_norm_fused_64(A.data_ptr(), W.data_ptr(), rms_gpu.data_ptr(), C.data_ptr(), M, N, eps, dim)
     _check("RMS_Norm_int64")
+    if not host_rms:
+        return (C, rms_gpu)
     rms[:M] = rms_gpu[:M].cpu()
     return (C, rms)
 
 
-def RMS_Norm_residual_int64(X: torch.Tensor, Y: torch.Tensor, k: int, W: torch.Tensor, eps, dim, inplace=False):
+def RMS_Norm_residual_int64(X: torch.Tensor, Y: torch.Tensor, k: int, W: torch.Tensor, eps, dim, inplace=False, host_rms=True):
     """The residual connection and the norm behind it in one pass over the row (inference/model.py:1465-1468,
     1472 with the next block's :1453): X' = X + Y * 2^k in wrapping int64, C = RMSNorm(X') with weights W.
     Returns (X', C, rms buffer); inplace=True writes X' over X."""
@@ -282,6 +308,8 @@ def RMS_Norm_residual_int64(X: torch.Tensor, Y: torch.Tensor, k: int, W: torch.T
     fn = lib.rms_norm_residual_fused_32 if W.dtype == torch.int32 else lib.rms_norm_residual_fused_64
     fn(X.data_ptr(), Y.data_ptr(), k, W.data_ptr(), Xout.data_ptr(), rms_gpu.data_ptr(), C.data_ptr(), M, N, eps, dim)
     _check("RMS_Norm_residual_int64")
+    if not host_rms:
+        return (Xout, C, rms_gpu)
     rms[:M] = rms_gpu[:M].cpu()
     return (Xout, C, rms)
 
