@@ -155,13 +155,15 @@ def test_gemm_head_projection_divisor_on_mfma(K, oracle, w32, b_rs):
         A = rand_i64(rng, (1, M, 320), 36)
         for _ in range(2):                                     # the second call runs on the remembered digit counts
             _gemm_case(K, oracle, 0, A, W, 1, b_rs, 21)
-        # one or two rows take the matrix-vector kernel; 45-bit weights / 2 still need six digits
-        mfma_expected = 2 < M <= 32 and (w32 or b_rs >= 256)
+        # one or two rows take the matrix-vector kernel, up to 16 the 16-row MFMA tiles (any width: a wavefront that
+        # meets more than five digits recomputes on the vector ALU by itself), up to 32 the 32-row MFMA kernels, for
+        # which 45-bit weights / 2 still need six digits
+        mfma_expected = 2 < M <= 16 or (16 < M <= 32 and (w32 or b_rs >= 256))
         assert (K.gemm_last_plan()[0] == 2) == mfma_expected, (M, K.gemm_last_plan())
-    # the 32-row MFMA kernels on a single row, asked for by name
+    # the MFMA kernels on a single row, asked for by name
     A = rand_i64(rng, (1, 1, 320), 36)
     _gemm_case(K, oracle, 2, A, W, 1, b_rs, 21)
-    assert (K.gemm_last_plan()[0] == 2) == (w32 or b_rs >= 256)
+    assert K.gemm_last_plan()[0] == 2
     K.lib.zk_gemm_set_path(0)
 
 
@@ -204,6 +206,89 @@ def test_gemm_one_or_two_rows(K, oracle, M, w32):
     K._check("gemv")
     Ce, Re = oracle.int64_bmm_broadcast(Av, Wv, 1, 1, 17)
     assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+
+
+@pytest.mark.parametrize("w32", [False, True])
+@pytest.mark.parametrize("M", [1, 3, 8, 15, 16])
+def test_gemm_up_to_16_rows(K, oracle, M, w32):
+    """the 16-row MFMA tiles (every wavefront on its own, digit counts taken from each step's data): one K slice and
+    several (partial sums added atomically, the last slice finishes), ragged N and K, batches, every digit path from
+    (3,3) to (5,5), operands beyond five digits (the wavefronts that meet them recompute on the vector ALU), widths that
+    change from step to step, every shift class, with and without remainder"""
+    rng = np.random.default_rng(160 + M + w32)
+    K.lib.zk_gemm_set_path(2)
+    for Bd, Kd, N, bits_a, bits_w, c in ((1, 7168, 576, 20, 16, 29), (1, 2048, 7168, 28, 31, 30), (2, 333, 130, 37, 30, 0),
+                                         (1, 64, 20000, 31, 31, 16), (3, 1000, 50, 63, 63, 0), (1, 4100, 33, 63, 31, 63),
+                                         (1, 1, 1, 63, 63, 1), (1, 640, 700, 45, 20, 33), (5, 130, 31, 22, 22, 7)):
+        A = rand_i64(rng, (Bd, M, Kd), bits_a)
+        W = rand_i32(rng, (N, Kd), min(bits_w, 31)) if w32 else rand_i64(rng, (N, Kd), bits_w)
+        _gemm_case(K, oracle, 2, A, W, 1, 1, c)
+        assert K.gemm_last_plan() == (2, 0, 0)
+    # widths that differ from step to step and from column tile to column tile: narrow everywhere, four and five digits
+    # in places, and one element beyond five digits in a single step of a single row
+    Kd, N = 1024, 200
+    A = rand_i64(rng, (1, M, Kd), 20)
+    W = rand_i32(rng, (N, Kd), 16) if w32 else rand_i64(rng, (N, Kd), 16)
+    A[0, :, 128:192] = rand_i64(rng, (M, 64), 29)
+    A[0, M - 1, 300] = -(1 << 37)
+    W[40:56, 512:640] = (rand_i32(rng, (16, 128), 31) if w32 else rand_i64(rng, (16, 128), 37))
+    _gemm_case(K, oracle, 2, A, W, 1, 1, 23)
+    A[0, 0, 1000] = (1 << 62) + 12345
+    if not w32:
+        W[199, 7] = -(1 << 63)
+    _gemm_case(K, oracle, 2, A, W, 1, 1, 23)
+    # no remainder wanted; operand divisor on B
+    C, R = K.int64_bmm_broadcast(dev(A), dev(W), 1, 1, 23, want_remainder=False)
+    assert R is None and np.array_equal(host(C), oracle.int64_bmm_broadcast(A, W, 1, 1, 23)[0])
+    _gemm_case(K, oracle, 2, A, W, 1, 256, 11)
+    # digits at their extremes over many steps between two folds of the int32 accumulators
+    # (digits -128, -128, -128, -128, 63: the largest magnitudes among the values that take the five-digit path)
+    x5 = (63 << 32) - 0x80808080
+    A = np.full((1, M, 2048), x5, np.int64)
+    W = np.full((70, 2048), -(1 << 31), np.int32) if w32 else np.full((70, 2048), x5, np.int64)
+    W[1::2] = (1 << 31) - 1 if w32 else -x5
+    _gemm_case(K, oracle, 2, A, W, 1, 1, 40)
+    # rows that start 8 bytes off a 16-byte boundary: the element-wise loads
+    buf = torch.zeros((M * 301 + 1,), dtype=torch.int64, device="cuda")
+    Av = rand_i64(rng, (1, M, 301), 30)
+    Ad = buf[1:].view(1, M, 301)
+    Ad.copy_(dev(Av))
+    Wv = rand_i32(rng, (50, 301)) if w32 else rand_i64(rng, (50, 301), 30)
+    Wd = dev(Wv)
+    C = torch.empty((1, M, 50), dtype=torch.int64, device="cuda")
+    R = torch.empty_like(C)
+    fn = K.lib.int64_32_bmm_broadcast_launcher if w32 else K.lib.int64_64_bmm_broadcast_launcher
+    fn(Ad.data_ptr(), Wd.data_ptr(), C.data_ptr(), R.data_ptr(), 1, 1, 17, 1, M, 301, 50)
+    K._check("rows16")
+    Ce, Re = oracle.int64_bmm_broadcast(Av, Wv, 1, 1, 17)
+    assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+    # the per-head einsums on a few sequence positions: the heads as a strided batch of k-contiguous int32 matrices
+    H, D, Cc = 16, 24, 40
+    a = rand_i64(rng, (1, M, H, Cc), 30)
+    w = rand_i32(rng, (H, D, Cc), 25)
+    assert np.array_equal(host(K.einsum_bshc_hdc_bshd(dev(a), dev(w), 21)), oracle.einsum_bshc_hdc_bshd(a, w, 21))
+    assert K.gemm_last_plan() == (2, 0, 0)
+    # and the scores of a few positions against a cache: bshc,btc->bsht with S * H <= 16
+    qq = rand_i64(rng, (2, 1, M, 192), 30)
+    kk = rand_i64(rng, (2, 300, 192), 24)
+    assert np.array_equal(host(K.einsum_bshc_btc_bsht(dev(qq), dev(kk), 21)), oracle.einsum_bshc_btc_bsht(qq, kk, 21))
+    K.lib.zk_gemm_set_path(0)
+
+
+def test_gemm_split_k_scratch_is_left_zeroed(K, oracle):
+    """several K slices per output tile add into scratch that the last slice leaves zeroed: calls of different shapes one
+    after the other, asynchronously, must not see each other's partial sums"""
+    rng = np.random.default_rng(170)
+    K.lib.zk_gemm_set_path(2)
+    shapes = [(16, 7168, 576), (5, 4096, 64), (16, 7168, 576), (9, 2048, 1000), (3, 8192, 33)]
+    ops = [(rand_i64(rng, (1, M, Kd), 30), rand_i64(rng, (N, Kd), 33)) for M, Kd, N in shapes]
+    devs = [(dev(a), dev(w)) for a, w in ops]
+    outs = [K.int64_bmm_broadcast(a, w, 1, 1, 19) for a, w in devs for _ in range(2)]
+    for i, (a, w) in enumerate(ops):
+        Ce, Re = oracle.int64_bmm_broadcast(a, w, 1, 1, 19)
+        for C, R in outs[2 * i: 2 * i + 2]:
+            assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re), shapes[i]
+    K.lib.zk_gemm_set_path(0)
 
 
 @pytest.mark.parametrize("M", [1, 2])
@@ -770,7 +855,7 @@ def test_gemm_mfma_path_is_taken(K, oracle):
     K.lib.zk_gemm_set_path(0)
 
 
-@pytest.mark.parametrize("M", [16, 48])
+@pytest.mark.parametrize("M", [20, 48])
 def test_gemm_stale_digit_guess_is_caught(K, oracle, M):
     """Operands that change in place under the same pointers.  The call after the change runs on the digit
     counts remembered for those pointers and does not wait for their check; the guarded recomputation behind
@@ -1004,8 +1089,8 @@ def test_moe_dispatch_reports_indices_outside_the_experts(K, oracle):
 @pytest.mark.parametrize("bits", [(20, 16), (37, 30), (50, 31)])
 def test_int64_grouped_bmm(K, oracle, path, w32, bits):
     """one launch over all experts against the per-expert oracle GEMMs: empty experts, experts with more than 32
-    rows, ragged K and N, the remainder output; (50, 31)-bit operands are wider than the 32-row kernels take and go
-    expert by expert"""
+    rows, ragged K and N, the remainder output; (50, 31)-bit operands are wider than five digits, which the wavefronts
+    that meet them recompute on the vector ALU"""
     rng = np.random.default_rng(bits[0] + w32)
     T, E, Kr, Kd, N = 90, 12, 3, 200, 300
     idx = _routing(rng, T, E, Kr)
@@ -1025,8 +1110,7 @@ def test_int64_grouped_bmm(K, oracle, path, w32, bits):
         Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
         assert np.array_equal(host(C), Ce), "quotient"
         assert np.array_equal(host(R), Re), "remainder"
-    single_launch = path != 1 and bits[0] <= 39
-    assert K.lib.zk_gemm_grouped_mfma_calls() - before == (2 if single_launch else 0), "which route the product took"
+    assert K.lib.zk_gemm_grouped_mfma_calls() - before == (2 if path != 1 else 0), "which route the product took"
     K.lib.zk_gemm_set_path(0)
 
 

@@ -125,7 +125,7 @@ def test_stale_guess_fresh_activations_known_weights(K, oracle):
     rng = np.random.default_rng(11)
     W = Operand(rand_i32(rng, (700, 384), 30))
     keep = []                 # earlier activations stay alive, so every call sees an address it has not seen
-    for M in (40, 16):
+    for M in (40, 24):
         Ce = None
         for rep in range(3):
             a = rand_i64(rng, (1, M, 384), 20)
@@ -242,7 +242,7 @@ def test_stale_guess_split_tail_tiles_of_a_multi_round_launch(K, oracle):
 def test_stale_guess_divided_weights(K, oracle, w32):
     """the head projection's form: B divided by a power of two inside the 32-row kernels, tracked on the divided values"""
     rng = np.random.default_rng(71 + w32)
-    M, Kd, N = 8, 2048, 1100
+    M, Kd, N = 24, 2048, 1100
     A = Operand(rand_i64(rng, (1, M, Kd), 20))
     W = Operand(rand_i32(rng, (N, Kd), 24) if w32 else rand_i64(rng, (N, Kd), 24))
     # (an int32 weight divided by 256 needs a fourth digit only at the top of the positive range: three digits hold

@@ -39,6 +39,16 @@ bool gemm_gemv_launch(const GemmDesc &d);
 // error (recorded).  The outcome describes this call only, whatever the sticky error channel holds from earlier ones.
 int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 
+// A handful of rows (M <= 16) against k-contiguous B on the 16-row MFMA tiles: every wavefront on its own, digit counts
+// taken from the data (nothing guessed, nothing read back), K split over wavefronts when the launch would not fill the
+// device otherwise (a second, small launch then adds the slices' partial sums).  acc: scratch for those sums (`max_slots`
+// slots of 8 KB: one per output tile of 16 x 32 and workgroup of slices; nothing in it needs clearing); null: the library's
+// own, grown on demand.  Returns 0 when launched, 1 when the descriptor is outside what it takes (nothing launched), -1
+// on an error (recorded).
+int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc = nullptr, size_t max_slots = 0);
+size_t gemm_rows16_workspace_bytes();
+void gemm_rows16_release_workspace();
+
 // Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
 // vector-ALU recomputation (known once their range has reached the host).
 long gemm_mfma_guard_hits();
@@ -71,6 +81,9 @@ struct GroupedDesc {
 // Streams a B once per row of its segment, so it is for a handful of rows (a decoding step's routed experts).
 // Returns false (nothing launched) when the descriptor is outside what it takes.
 bool gemm_gemv_grouped_launch(const GroupedDesc &d);
+
+// The grouped product on the 16-row MFMA tiles (see gemm_rows16_launch): one launch, no wait.  0 / 1 / -1 as there.
+int gemm_rows16_grouped(const GroupedDesc &d);
 
 // One launch of the 32-row-tile MFMA kernels over all groups.  Returns 0 when done, 1 when the operands need
 // more digits than those kernels are built for (nothing valid was written: the caller takes another route),

@@ -23,6 +23,16 @@ bool gemm_dispatch(const char *name, const GemmDesc &d)
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
         return check_launch(name);
     }
+    // up to 16 rows against k-contiguous weights: the 16-row MFMA tiles, digit counts taken from the data on the device
+    // (prepared weights keep the kernels that read their planes: fewer bytes per weight)
+    if (g_gemm_path != kPathValu && !gemm_mfma_is_prepared(d.B)) {
+        const int rc = gemm_rows16_launch(d);
+        if (rc == 0) {
+            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0;
+            return check_launch(name);
+        }
+        if (rc < 0) return false;
+    }
     if (g_gemm_path != kPathValu) {
         int la = 0, lb = 0;
         // 0: launched, 1: declined (whatever the error channel holds comes from an earlier call and must not keep this
@@ -59,6 +69,16 @@ void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
         g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
         check_launch(name);
         return;
+    }
+    if (g_gemm_path != kPathValu && !gemm_mfma_is_prepared((const void *)d.B)) {
+        const int rc = gemm_rows16_grouped(d);
+        if (rc == 0) {
+            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0;
+            g_grouped_mfma_calls++;
+            check_launch(name);
+            return;
+        }
+        if (rc < 0) return;
     }
     if (g_gemm_path != kPathValu && d.K > 0) {
         int la = 0, lb = 0;

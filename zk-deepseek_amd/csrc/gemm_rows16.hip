@@ -1,0 +1,681 @@
+// GEMM for a handful of rows (M <= 16 per row tile): weight streams on v_mfma_i32_16x16x64_i8, every wavefront on
+// its own, digit counts taken from the data.
+//
+// A product of a few activation rows with a wide weight matrix (the MLA down-projections on a short prompt, the routed
+// experts of a MoE layer with ~8 tokens each) is bound by the one pass over the weights, and the 32-row tiles of the
+// general kernel multiply mostly padding there.  This kernel uses the 16x16x64 i8 MFMA, whose operand fragment is 16
+// bytes of ONE row per lane: lane (i, q) = (lane % 16, lane / 16) holds 16 of the 64 k of a step for row i.  A lane can
+// therefore load its own fragment straight from global memory (eight 16-byte loads for int64, four for int32 weights;
+// the four lanes of a row read 64 contiguous bytes per load), split it into balanced base-256 digits in registers
+// (see gemm_mfma.hip for the digit scheme) and feed the matrix pipe: no LDS, no barrier, no cooperation between
+// wavefronts.  Which k a fragment byte stands for does not matter as long as both operands agree, so the byte order
+// follows the loads.
+//
+// Nothing is guessed.  Before a step is split, the wavefront ORs the magnitudes of what it loaded and picks the digit
+// counts that step needs (3, 4 or 5 per operand, accumulated in nine int32 diagonals per tile).  A wavefront that
+// meets values beyond five digits (2^38 and up: nothing a model produces) drops what it has and recomputes its
+// outputs with 128-bit multiply-adds on the vector ALU.  Results are exact for every input, no range travels to the
+// host, and the call never waits.
+//
+// A work item is (batch or expert, 16-row tile, group of 32 columns, slice of K); one wavefront = one workgroup = one
+// item, four wavefronts to a workgroup.  With one slice the wavefront stores C and R itself.  With several (a launch too
+// small to fill the device otherwise), the four wavefronts of a workgroup are four slices of one tile: they add up in
+// LDS, the workgroup leaves its 128-bit sums in a slot of scratch and takes a ticket, and the workgroup that arrives
+// last adds the slots, applies rounding term and shift, stores, and resets the ticket for the next call.
+#include "gemm_mfma_kernels.h"
+
+namespace zk {
+
+struct Rows16Params {
+    const int64_t *A;
+    const void *B;
+    int64_t *C, *R;
+    long lda, sA, ldb, sB, ldc, sC;      // element strides: A[g*sA + m*lda + k], B[g*sB + n*ldb + k]
+    int G, M, N, K, shift, b_shift;
+    int64_t init;
+    int row_tiles, col_groups, nslices;
+    unsigned long long *acc;             // split K: per (g, row tile, column group) and workgroup of slices, the workgroup's 128-bit sums
+    // grouped mode: rows of A and C form one segment per group, every group has its own B (see GroupedDesc)
+    const int *grp_seg, *grp_tiles, *grp_ntiles;
+    const void *const *grp_b;
+    int dbg;
+};
+
+constexpr int kR16Fast = 9;              // diagonals the accumulators hold: digit pairs up to (5, 5)
+constexpr int kR16FoldSteps = 16;        // steps between folds of the accumulators (5 pairs * 64 * 2^14 * 16 < 2^31)
+constexpr int kR16Waves = 4;             // wavefronts per workgroup (one per SIMD: the kernel takes most of the register file)
+constexpr int kR16RingBytes = 32 * 1024; // LDS per wavefront: the ring of steps on their way from HBM
+
+// 16-column tiles per wavefront: a step of int32 weights is half the bytes of a step of int64 weights
+template <bool B32> struct R16Shape {
+    static constexpr int kColTiles = B32 ? 2 : 1;
+    static constexpr int kCols = 16 * kColTiles;
+    static constexpr int kLoadsPerTile = B32 ? 4 : 8;                       // 16-byte loads per lane and column tile
+    static constexpr int kStageBytes = (8 + kColTiles * kLoadsPerTile) * 1024;   // A's eight loads, then the tiles'
+    static constexpr int kStages = kR16RingBytes / kStageBytes;
+    static_assert(kStages >= 2, "the ring holds at least two steps");
+};
+
+// ---- loads that bypass the registers ------------------------------------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS: one wave-instruction fills
+// 1 KB at a wave-uniform base (M0), lane l at byte 16 l.  The compiler does not know that these instructions load or
+// that they write LDS, so the waits are explicit: vector-memory loads of a wave complete in order, and "at most N
+// outstanding" with N = the loads issued since guarantees that everything older has landed.
+__device__ __forceinline__ void lds_dma16(const void *gptr, unsigned lds_base)
+{
+    // (the base is the same in every lane, but derived from the wavefront's number, which the compiler holds in a vector register)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));      // expcnt and lgkmcnt left at their maxima
+}
+
+// ---- digit split of a fragment (16 elements of one row) ----------------------------------------------------
+// 64-bit elements, any digit count: two groups of 8, k ascending within the fragment
+template <int N>
+__device__ __forceinline__ void split16(const int64_t (&x)[16], v4i (&out)[N])
+{
+    uint2 a[N], b[N];
+    limb_split8<N>(*reinterpret_cast<const int64_t(*)[8]>(&x[0]), a);
+    limb_split8<N>(*reinterpret_cast<const int64_t(*)[8]>(&x[8]), b);
+#pragma unroll
+    for (int i = 0; i < N; i++) out[i] = v4i{ (int)a[i].x, (int)a[i].y, (int)b[i].x, (int)b[i].y };
+}
+
+// Elements that fit 32 bits.  N <= 4: x + bias stays inside 32 bits (the caller has checked |x| < 2^(8N-2)), the digits
+// are its bytes.  N == 5 (any int32): the fifth digit is the carry of the biased sum of a non-negative element.
+template <int N>
+__device__ __forceinline__ void split16_w32(const int (&x)[16], v4i (&out)[N])
+{
+    constexpr uint32_t bias = N >= 5 ? 0x80808080u : (0x00808080u >> (8 * (4 - N)));
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        uint32_t y[4], o[4], e = 0;
+#pragma unroll
+        for (int z = 0; z < 4; z++) {
+            const uint32_t xv = (uint32_t)x[4 * w + z], u = xv + bias;
+            if (N >= 5) e |= ((u < bias && x[4 * w + z] >= 0) ? 1u : 0u) << (8 * z);
+            y[z] = u ^ bias;
+        }
+        transpose4(y[0], y[1], y[2], y[3], o);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < N) out[i][w] = (int)o[i];
+        if (N >= 5) out[4][w] = (int)e;
+    }
+}
+
+// The 64 k of a step are dealt to (lane quarter q, fragment byte b) so that every load is 16 bytes and the four lanes
+// of a row read 64 contiguous bytes:
+//   int64 weights: byte b <-> k = 8*(b/2) + 2*q + b%2      (A and B: eight loads of two elements)
+//   int32 weights: byte b <-> k = 16*(b/4) + 4*q + b%4     (B: four loads of four elements; A: eight loads of two)
+template <bool B32>
+__device__ __forceinline__ int frag_k(int q, int b) { return B32 ? 16 * (b >> 2) + 4 * q + (b & 3) : 8 * (b >> 1) + 2 * q + (b & 1); }
+
+// sums[r] += sum_d acc[d][r] * 2^(8 d): diagonals in groups of four (a group stays below 2^57), the groups meet in 128 bits
+template <int D>
+__device__ __forceinline__ void fold_diagonals(const v4i (&acc)[D], u128 (&sums)[4])
+{
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+#pragma unroll
+        for (int gq = 0; gq < (D + 3) / 4; gq++) {
+            uint64_t s = (uint64_t)(int64_t)acc[4 * gq][r];
+#pragma unroll
+            for (int j = 1; j < 4; j++)
+                if (4 * gq + j < D) s += (uint64_t)(int64_t)acc[4 * gq + j][r] << (8 * j);
+            sums[r] += (u128)(i128)(int64_t)s << (32 * gq);
+        }
+    }
+}
+
+// One operand fragment as loaded: 16 elements of 64 bits (A, int64 weights) or of 32 bits (int32 weights), as the
+// 16-byte pieces the loads delivered.
+template <bool W32> struct RawFrag { v4i v[W32 ? 4 : 8]; };
+
+template <bool W32>
+__device__ __forceinline__ uint64_t magnitude_or(const RawFrag<W32> &f)
+{
+    // OR of x for x >= 0 and ~x otherwise: below 2^(8n-2) means n digits hold every element
+    if (W32) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int z = 0; z < 4; z++) m |= (uint32_t)(f.v[j][z] ^ (f.v[j][z] >> 31));
+        return m;
+    }
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int s = f.v[j][2 * h + 1] >> 31;
+            lo |= (uint32_t)(f.v[j][2 * h] ^ s);
+            hi |= (uint32_t)(f.v[j][2 * h + 1] ^ s);
+        }
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// digits (3, 4, 5, or 9 for "more") that hold every element of the wavefront whose magnitudes OR to m in some lane
+__device__ __forceinline__ int wave_digits(uint64_t m)
+{
+    if (__builtin_amdgcn_ballot_w64(m >> 22 != 0) == 0) return 3;
+    if (__builtin_amdgcn_ballot_w64(m >> 30 != 0) == 0) return 4;
+    if (__builtin_amdgcn_ballot_w64(m >> 38 != 0) == 0) return 5;
+    return 9;
+}
+
+template <int N, bool W32>
+__device__ __forceinline__ void split_frag(const RawFrag<W32> &f, v4i (&out)[N])
+{
+    if (W32) {
+        int x[16];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int z = 0; z < 4; z++) x[4 * j + z] = f.v[j][z];
+        split16_w32<N>(x, out);
+    } else if (N <= 4) {
+        int x[16];                  // values below 2^(8N-2): the low words say it all
+#pragma unroll
+        for (int j = 0; j < 8; j++) { x[2 * j] = f.v[j][0]; x[2 * j + 1] = f.v[j][2]; }
+        split16_w32<N>(x, out);
+    } else {
+        int64_t x[16];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            x[2 * j] = (int64_t)(((uint64_t)(uint32_t)f.v[j][1] << 32) | (uint32_t)f.v[j][0]);
+            x[2 * j + 1] = (int64_t)(((uint64_t)(uint32_t)f.v[j][3] << 32) | (uint32_t)f.v[j][2]);
+        }
+        split16<N>(x, out);
+    }
+}
+
+template <int NA, int NB, bool B32>
+__device__ __forceinline__ void step_fast(const RawFrag<false> &fa_raw, const RawFrag<B32> (&fw_raw)[R16Shape<B32>::kColTiles],
+                                          v4i (&acc)[R16Shape<B32>::kColTiles][kR16Fast])
+{
+    v4i fa[NA];
+    split_frag<NA, false>(fa_raw, fa);
+#pragma unroll
+    for (int ct = 0; ct < R16Shape<B32>::kColTiles; ct++) {
+        v4i fb[NB];
+        split_frag<NB, B32>(fw_raw[ct], fb);
+#pragma unroll
+        for (int i = 0; i < NA; i++)
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                acc[ct][i + j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[i], fb[j], acc[ct][i + j], 0, 0, 0);
+    }
+}
+
+template <bool B32, bool GRP>
+__global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Params p)
+{
+    typedef R16Shape<B32> S;
+    constexpr int CT = S::kColTiles, LPT = S::kLoadsPerTile, LPS = 8 + CT * LPT;     // loads per lane and step
+    extern __shared__ __attribute__((aligned(16))) unsigned char r16_smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, q = lane >> 4;
+    unsigned char *ring = r16_smem + wave * kR16RingBytes;
+    const unsigned ring_lds = (unsigned)(uintptr_t)ring;             // LDS byte address of this wavefront's ring
+
+    // wavefront -> item (batch or 32-row tile half, column group, K slice).  With several slices the slice moves fastest:
+    // the wavefronts of a workgroup are then four slices of one output tile and add up in LDS first.  Otherwise the
+    // column group does: the wavefronts that run side by side share their rows of A.
+    unsigned item = blockIdx.x * kR16Waves + wave;                 // (the host keeps the item count below 2^31)
+    int slice = 0;
+    if (p.nslices > 1) { slice = (int)(item % (unsigned)p.nslices); item /= (unsigned)p.nslices; }
+    const int cg = (int)(item % (unsigned)p.col_groups);
+    item /= (unsigned)p.col_groups;
+    int g = 0, m0 = 0, m_lim = p.M;
+    const void *b_base = p.B;
+    long tile_id = 0;                       // index of (g, row tile, column group) among the launch's output tiles
+    bool live = true;
+    if (GRP) {
+        // item = (32-row tile of the dispatch table, half): 16 rows each
+        const int mt = (int)(item >> 1), half = (int)(item & 1);
+        live = mt < *p.grp_ntiles;
+        if (live) {
+            const int e = p.grp_tiles[2 * mt];
+            m0 = p.grp_tiles[2 * mt + 1] + 16 * half;
+            m_lim = p.grp_seg[e + 1];
+            live = m0 < m_lim;
+            b_base = p.grp_b[e];
+        }
+    } else {
+        const int rt = (int)(item % (unsigned)p.row_tiles);
+        g = (int)(item / (unsigned)p.row_tiles);
+        live = g < p.G;
+        m0 = rt * 16;
+        tile_id = ((long)g * p.row_tiles + rt) * p.col_groups + cg;
+    }
+    if (!live) return;                      // (only without K slices: no barrier lies ahead)
+    const int n0 = cg * S::kCols;
+
+    // this lane's rows (clamped: the products of rows past the end land in outputs that are never stored)
+    int am = m0 + li;
+    am = am < m_lim ? am : m_lim - 1;
+    const int64_t *a_row = p.A + (long)g * p.sA + (long)am * p.lda;
+    const char *w_row[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) {
+        int n = n0 + 16 * ct + li;
+        n = n < p.N ? n : p.N - 1;
+        w_row[ct] = reinterpret_cast<const char *>(b_base) + ((long)g * p.sB + (long)n * p.ldb) * (B32 ? 4 : 8);
+    }
+    const bool vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0 &&
+                     (((uintptr_t)b_base | (uintptr_t)(p.ldb * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
+
+    const int ksteps = (p.K + 63) / 64;
+    const int ks_begin = (int)((long)slice * ksteps / p.nslices), ks_end = (int)((long)(slice + 1) * ksteps / p.nslices);
+    // steps that travel through the ring: whole ones, on 16-byte aligned rows; the others are loaded element by element
+    const int full_end = vec ? (p.K / 64 < ks_end ? p.K / 64 : ks_end) : ks_begin;
+
+    v4i acc[CT][kR16Fast];
+    u128 sums[CT][4];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+        for (int d = 0; d < kR16Fast; d++) acc[ct][d] = v4i{ 0, 0, 0, 0 };
+#pragma unroll
+        for (int r = 0; r < 4; r++) sums[ct][r] = 0;
+    }
+    auto fold = [&]() {
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            fold_diagonals<kR16Fast>(acc[ct], sums[ct]);
+#pragma unroll
+            for (int d = 0; d < kR16Fast; d++) acc[ct][d] = v4i{ 0, 0, 0, 0 };
+        }
+    };
+
+    // stage `st` of the ring <- step ks: A's eight pieces, then every tile's
+    auto issue = [&](int ks, int st) {
+        const int k0 = ks * 64;
+        const unsigned base = ring_lds + st * S::kStageBytes;
+#pragma unroll
+        for (int j = 0; j < 8; j++) if (!(p.dbg & 4) || j < 1) lds_dma16(a_row + k0 + frag_k<B32>(q, 2 * j), base + j * 1024); else lds_dma16(a_row, base + j * 1024);
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int j = 0; j < LPT; j++) {
+                if (p.dbg & 8) {
+                    // bandwidth experiment: each instruction reads whole 256-byte (int32) / 512-byte runs of a row
+                    const int rows_per = B32 ? 4 : 2, lanes_per = 64 / rows_per;
+                    int n = n0 + 16 * ct + rows_per * j + lane / lanes_per;
+                    n = n < p.N ? n : p.N - 1;
+                    const char *rowp = reinterpret_cast<const char *>(b_base) + ((long)g * p.sB + (long)n * p.ldb) * (B32 ? 4 : 8);
+                    lds_dma16(rowp + (long)k0 * (B32 ? 4 : 8) + (lane % lanes_per) * 16, base + (8 + ct * LPT + j) * 1024);
+                } else
+                lds_dma16(w_row[ct] + (long)(k0 + frag_k<B32>(q, (16 / LPT) * j)) * (B32 ? 4 : 8), base + (8 + ct * LPT + j) * 1024);
+            }
+    };
+
+    RawFrag<false> fa;
+    RawFrag<B32> fw[CT];
+    int since_fold = 0;
+    bool wide = false;
+    // one step on the fragments in fa / fw: digit counts from the data, split, multiply
+    auto process = [&]() {
+        if (p.b_shift) {
+            // weights divided by a power of two first (truncating toward zero)
+#pragma unroll
+            for (int ct = 0; ct < CT; ct++) {
+                if (B32) {
+#pragma unroll
+                    for (int j = 0; j < LPT; j++)
+#pragma unroll
+                        for (int z = 0; z < 4; z++) fw[ct].v[j][z] = (int)tdiv_pow2((int64_t)fw[ct].v[j][z], p.b_shift > 31 ? 31 : p.b_shift);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < LPT; j++)
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const int64_t x = (int64_t)(((uint64_t)(uint32_t)fw[ct].v[j][2 * h + 1] << 32) | (uint32_t)fw[ct].v[j][2 * h]);
+                            const int64_t y = tdiv_pow2(x, p.b_shift);
+                            fw[ct].v[j][2 * h] = (int)(uint32_t)y;
+                            fw[ct].v[j][2 * h + 1] = (int)(uint32_t)((uint64_t)y >> 32);
+                        }
+                }
+            }
+        }
+        uint64_t mw = 0;
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) mw |= magnitude_or<B32>(fw[ct]);
+        const int na = wave_digits(magnitude_or<false>(fa));
+        int nb = wave_digits(mw);
+        if (B32 && nb > 5) nb = 5;                          // (an int32 never needs more)
+        if (na > 5 || nb > 5) { wide = true; return; }
+        switch ((na - 3) * 3 + (nb - 3)) {
+        case 0: step_fast<3, 3, B32>(fa, fw, acc); break;
+        case 1: step_fast<3, 4, B32>(fa, fw, acc); break;
+        case 2: step_fast<3, 5, B32>(fa, fw, acc); break;
+        case 3: step_fast<4, 3, B32>(fa, fw, acc); break;
+        case 4: step_fast<4, 4, B32>(fa, fw, acc); break;
+        case 5: step_fast<4, 5, B32>(fa, fw, acc); break;
+        case 6: step_fast<5, 3, B32>(fa, fw, acc); break;
+        case 7: step_fast<5, 4, B32>(fa, fw, acc); break;
+        default: step_fast<5, 5, B32>(fa, fw, acc); break;
+        }
+        if (++since_fold == kR16FoldSteps) { fold(); since_fold = 0; }
+    };
+
+    // the ring: up to kStages steps under way; a stage is refilled as soon as its step sits in registers
+#pragma unroll
+    for (int st = 0; st < S::kStages; st++)
+        if (ks_begin + st < full_end && !(p.dbg & 2)) issue(ks_begin + st, st);
+    int st = 0;
+    for (int ks = ks_begin; ks < full_end && !wide; ks++) {
+        // everything issued after step ks: the steps ks+1 .. ks+kStages-1 that exist
+        const int behind = full_end - 1 - ks < S::kStages - 1 ? full_end - 1 - ks : S::kStages - 1;
+        if (behind >= S::kStages - 1) wait_vmcnt<(S::kStages - 1) * LPS>();
+        else if (S::kStages > 2 && behind == S::kStages - 2) wait_vmcnt<(S::kStages > 2 ? S::kStages - 2 : 0) * LPS>();
+        else wait_vmcnt<0>();
+        const unsigned char *src = ring + st * S::kStageBytes + lane * 16;
+#pragma unroll
+        for (int j = 0; j < 8; j++) fa.v[j] = *reinterpret_cast<const v4i *>(src + j * 1024);
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int j = 0; j < LPT; j++) fw[ct].v[j] = *reinterpret_cast<const v4i *>(src + (8 + ct * LPT + j) * 1024);
+        if (ks + S::kStages < full_end) {
+            // (the reads above must have returned before the stage is overwritten)
+            __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0)
+            if (!(p.dbg & 2)) issue(ks + S::kStages, st);
+        }
+        st = st + 1 == S::kStages ? 0 : st + 1;
+        if (!(p.dbg & 1)) process();
+    }
+    wait_vmcnt<0>();
+    // steps outside the ring (a partial last step, rows that are not 16-byte aligned): element by element
+    for (int ks = full_end; ks < ks_end && !wide; ks++) {
+        const int k0 = ks * 64, k_left = p.K - k0;
+#pragma unroll
+        for (int b = 0; b < 16; b++) {
+            const int k = frag_k<B32>(q, b);
+            const int64_t x = k < k_left ? a_row[k0 + k] : 0;
+            fa.v[b >> 1][2 * (b & 1)] = (int)(uint32_t)x;
+            fa.v[b >> 1][2 * (b & 1) + 1] = (int)(uint32_t)((uint64_t)x >> 32);
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int b = 0; b < 16; b++) {
+                const int k = frag_k<B32>(q, b);
+                if (B32) {
+                    fw[ct].v[b >> 2][b & 3] = k < k_left ? reinterpret_cast<const int32_t *>(w_row[ct])[k0 + k] : 0;
+                } else {
+                    const int64_t x = k < k_left ? reinterpret_cast<const int64_t *>(w_row[ct])[k0 + k] : 0;
+                    fw[ct].v[b >> 1][2 * (b & 1)] = (int)(uint32_t)x;
+                    fw[ct].v[b >> 1][2 * (b & 1) + 1] = (int)(uint32_t)((uint64_t)x >> 32);
+                }
+            }
+        process();
+    }
+    fold();
+    if (wide) {
+        // Values beyond five digits (2^38) somewhere in this item's slice: every lane recomputes its outputs with
+        // 128-bit multiply-adds on the vector ALU, straight from memory.  Slow and exact; model data never comes here.
+#pragma unroll 1
+        for (int o = 0; o < CT * 4; o++) {
+            const int ct = o >> 2, r = o & 3;
+            int m = m0 + 4 * q + r, n = n0 + 16 * ct + li;
+            m = m < m_lim ? m : m_lim - 1;
+            n = n < p.N ? n : p.N - 1;
+            const int64_t *ar = p.A + (long)g * p.sA + (long)m * p.lda;
+            const char *wr = reinterpret_cast<const char *>(b_base) + ((long)g * p.sB + (long)n * p.ldb) * (B32 ? 4 : 8);
+            const int k_end = ks_end * 64 < p.K ? ks_end * 64 : p.K;
+            u128 s = 0;
+            for (int k = ks_begin * 64; k < k_end; k++) {
+                int64_t w = B32 ? (int64_t)reinterpret_cast<const int32_t *>(wr)[k] : reinterpret_cast<const int64_t *>(wr)[k];
+                if (p.b_shift) w = tdiv_pow2(w, p.b_shift);
+                s += (u128)((i128)ar[k] * (i128)w);
+            }
+            // (static register indices: the sums stay in registers)
+#pragma unroll
+            for (int c2 = 0; c2 < CT; c2++)
+#pragma unroll
+                for (int r2 = 0; r2 < 4; r2++)
+                    if (c2 == ct && r2 == r) sums[c2][r2] = s;
+        }
+    }
+
+    // accumulator register r of lane (li, q) holds row 4*q + r, column li of its 16x16 tile
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+    auto store = [&](int ct, int r, uint64_t lo, uint64_t hi) {
+        const int m = m0 + 4 * q + r, n = n0 + 16 * ct + li;
+        const long o = (long)g * p.sC + (long)m * p.ldc + n;
+        p.C[o] = (int64_t)((lo >> p.shift) | ((hi << 1) << (63 - p.shift)));
+        if (p.R) p.R[o] = (int64_t)(lo & rmask);
+    };
+    if (p.nslices == 1) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (m0 + 4 * q + r >= m_lim || n0 + 16 * ct + li >= p.N) continue;
+                const u128 s = sums[ct][r] + (u128)(i128)p.init;
+                store(ct, r, (uint64_t)s, (uint64_t)(s >> 64));
+            }
+        return;
+    }
+    // Several slices.  The four wavefronts of the workgroup hold four slices of one tile: they meet in LDS (the rings are
+    // idle by now), the first one adds the workgroup's sums into the tile's zeroed scratch and counts in, and the
+    // workgroup that arrives last finishes the tile.
+    u128 *meet = reinterpret_cast<u128 *>(r16_smem);              // [wave][output][lane]
+    if (p.dbg & 64) return;
+    __syncthreads();
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) meet[(wave * (CT * 4) + ct * 4 + r) * 64 + lane] = sums[ct][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int w = 1; w < kR16Waves; w++) sums[ct][r] += meet[(w * (CT * 4) + ct * 4 + r) * 64 + lane];
+    // the workgroup's sums go to its own slot of the tile's scratch; a second launch adds the slots up
+    // (Finishing inside this kernel was measured first.  Adding into one slot with atomics: fourteen workgroups adding 512
+    // sums each spent 3.4 us in dependent round trips to the memory side, and every further slice 0.3 us.  A ticket with
+    // the last arriver adding the slots: a round trip for the stores, one for the ticket, and several for the loads,
+    // since nothing that crosses the dies may be fenced or cached.  A launch boundary costs less than either.)
+    const int groups = p.nslices / kR16Waves, grp = slice / kR16Waves;
+    u128 *slot = reinterpret_cast<u128 *>(p.acc) + ((long)tile_id * groups + grp) * (CT * 4 * 64);
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) slot[(ct * 4 + r) * 64 + lane] = sums[ct][r];
+}
+
+// Adds the slots of every output tile, applies rounding term and shift, stores C and R: one thread per output.
+template <bool B32>
+__global__ __launch_bounds__(256) void gemm_rows16_finish_kernel(Rows16Params p)
+{
+    constexpr int CT = R16Shape<B32>::kColTiles, PER = CT * 4 * 64;         // sums per slot
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long tile_id = idx / PER;
+    const int o = (int)(idx - tile_id * PER), lane = o & 63, cr = o >> 6, ct = cr >> 2, r = cr & 3;
+    const long tiles = (long)p.G * p.row_tiles * p.col_groups;
+    if (tile_id >= tiles) return;
+    const int cg = (int)(tile_id % p.col_groups);
+    const long t2 = tile_id / p.col_groups;
+    const int rt = (int)(t2 % p.row_tiles), g = (int)(t2 / p.row_tiles);
+    const int m = rt * 16 + 4 * (lane >> 4) + r, n = cg * R16Shape<B32>::kCols + 16 * ct + (lane & 15);
+    if (m >= p.M || n >= p.N) return;
+    const int groups = p.nslices / kR16Waves;
+    const u128 *slot = reinterpret_cast<const u128 *>(p.acc) + tile_id * groups * PER + o;
+    u128 s = (u128)(i128)p.init;
+#pragma unroll 8
+    for (int gi = 0; gi < groups; gi++) s += slot[(long)gi * PER];
+    const uint64_t lo = (uint64_t)s, hi = (uint64_t)(s >> 64);
+    const long at = (long)g * p.sC + (long)m * p.ldc + n;
+    p.C[at] = (int64_t)((lo >> p.shift) | ((hi << 1) << (63 - p.shift)));
+    if (p.R) p.R[at] = (int64_t)(p.shift ? lo & ((1ull << p.shift) - 1) : 0);
+}
+
+}  // namespace zk
+
+namespace zk {
+
+// ---- host side ---------------------------------------------------------------------------------------------
+// Scratch of the split-K launches, kept between calls: slots of 8 KB (the 128-bit sums of one workgroup for one output
+// tile).  Every slot a launch reads has been written by that launch: nothing needs clearing.
+static unsigned long long *g_r16_acc = nullptr;
+static size_t g_r16_slots = 0;
+static int g_r16_cus = 0;
+
+constexpr size_t kR16SlotBytes = 8 * 64 * 16;
+
+size_t gemm_rows16_workspace_bytes() { return g_r16_slots * kR16SlotBytes; }
+
+void gemm_rows16_release_workspace()
+{
+    if (g_r16_acc) (void)hipFree(g_r16_acc);
+    g_r16_acc = nullptr;
+    g_r16_slots = 0;
+}
+
+static int r16_cus()
+{
+    if (!g_r16_cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        g_r16_cus = n;
+    }
+    return g_r16_cus;
+}
+
+// 0: the buffer holds `slots` slots, 1: no memory (the caller runs without split K), -1: error recorded
+static int r16_scratch(size_t slots)
+{
+    if (slots <= g_r16_slots) return 0;
+    // the old buffer may still be in use by launches under way: the stream is drained first (this happens a few times
+    // in a process, while the largest launch is still growing)
+    if (g_r16_slots && hipStreamSynchronize(0) != hipSuccess) { set_error(kLaunchFailure, "gemm: cannot wait for the stream"); return -1; }
+    gemm_rows16_release_workspace();
+    if (hipMalloc(&g_r16_acc, slots * kR16SlotBytes) != hipSuccess) {
+        (void)hipGetLastError();
+        g_r16_acc = nullptr;
+        return 1;
+    }
+    g_r16_slots = slots;
+    return 0;
+}
+
+// How many slices of K per output tile.  One workgroup (four wavefronts) fits a compute unit, so a launch runs in
+// rounds of `cus` workgroups; the slices are a multiple of four (a workgroup's wavefronts add up in LDS before they touch
+// the scratch) and the count that minimises rounds x steps per wavefront wins, a split being charged the second launch.
+static int r16_slices(long tiles, int K, int cus)
+{
+    const int ksteps = (K + 63) / 64;
+    // in units of one step of one wavefront (about a microsecond): start-up of a round, the finishing launch
+    const double round_cost = 3.0, finish_cost = 4.0;
+    int best = 1;
+    double best_cost = 0;
+    for (int n = 1; n <= ksteps / 2 || n == 1; n = n == 1 ? kR16Waves : n + kR16Waves) {
+        const long wgs = (tiles * n + kR16Waves - 1) / kR16Waves;
+        const long rounds = (wgs + cus - 1) / cus;
+        const double cost = rounds * ((double)((ksteps + n - 1) / n) + round_cost) + (n > 1 ? finish_cost : 0.0);
+        if (n == 1 || cost < best_cost) { best = n; best_cost = cost; }
+    }
+    return best;
+}
+
+static bool r16_fill(const GemmDesc &d, Rows16Params &p)
+{
+    if (d.a_rs != 1 || d.ldbk != 1 || d.M < 1 || d.M > 16 || d.N < 1 || d.K < 0 || d.G < 1) return false;
+    int b_shift = 0;
+    if (d.b_rs != 1) {
+        if (d.b_rs <= 0 || (d.b_rs & (d.b_rs - 1)) != 0) return false;
+        while (((int64_t)1 << b_shift) < d.b_rs) b_shift++;
+    }
+    const int cols = d.b32 ? R16Shape<true>::kCols : R16Shape<false>::kCols;
+    p = Rows16Params{};
+    p.A = d.A; p.B = d.B; p.C = d.C; p.R = d.R;
+    p.lda = d.lda; p.sA = d.sA; p.ldb = d.ldbn; p.sB = d.sB; p.ldc = d.ldc; p.sC = d.sC;
+    p.G = d.G; p.M = d.M; p.N = d.N; p.K = d.K; p.shift = d.shift; p.b_shift = b_shift; p.init = d.init;
+    p.row_tiles = (d.M + 15) / 16;
+    p.col_groups = (d.N + cols - 1) / cols;
+    p.nslices = 1;
+    p.dbg = getenv("ZK_R16_DBG") ? atoi(getenv("ZK_R16_DBG")) : 0;
+    return true;
+}
+
+typedef void (*Rows16Kernel)(Rows16Params);
+
+static int r16_run(Rows16Kernel fn, const Rows16Params &p, long items)
+{
+    const long blocks = (items + kR16Waves - 1) / kR16Waves;
+    if (items > 0x7FFFFFF0L) return 1;
+    constexpr int lds = kR16Waves * kR16RingBytes;
+    static const void *raised[4] = {};
+    bool seen = false;
+    for (const void *f : raised) seen = seen || f == (const void *)fn;
+    if (!seen) {
+        if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+            set_error(kLaunchFailure, "gemm: cannot raise the LDS limit of the 16-row kernel to %d bytes", lds);
+            return -1;
+        }
+        for (const void *&f : raised)
+            if (!f) { f = (const void *)fn; break; }
+    }
+    fn<<<dim3((unsigned)blocks), dim3(64 * kR16Waves), lds, 0>>>(p);
+    if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: the 16-row kernel could not be launched"); return -1; }
+    return 0;
+}
+
+// acc: scratch for split K (`max_slots` slots of 8 KB); null: the library's own, grown on demand
+int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_slots)
+{
+    Rows16Params p;
+    if (!r16_fill(d, p)) return 1;
+    const long tiles = (long)d.G * p.row_tiles * p.col_groups;
+    if (tiles > (1L << 24)) return 1;
+    const int slices = r16_slices(tiles, d.K, r16_cus());
+    if (slices > 1) {
+        const size_t slots = (size_t)tiles * (slices / kR16Waves);
+        if (acc) {
+            if (slots <= max_slots) { p.acc = acc; p.nslices = slices; }
+        } else {
+            const int rc = r16_scratch(slots);
+            if (rc < 0) return -1;
+            if (rc == 0) { p.acc = g_r16_acc; p.nslices = slices; }
+        }
+    }
+    const int rc = r16_run(d.b32 ? gemm_rows16_kernel<true, false> : gemm_rows16_kernel<false, false>, p, tiles * p.nslices);
+    if (rc != 0 || p.nslices == 1) return rc;
+    const long threads = tiles * (d.b32 ? R16Shape<true>::kColTiles : R16Shape<false>::kColTiles) * 4 * 64;
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (d.b32) gemm_rows16_finish_kernel<true><<<grid, dim3(256), 0, 0>>>(p);
+    else gemm_rows16_finish_kernel<false><<<grid, dim3(256), 0, 0>>>(p);
+    if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: the finishing kernel could not be launched"); return -1; }
+    return 0;
+}
+
+int gemm_rows16_grouped(const GroupedDesc &d)
+{
+    if (d.K < 0 || d.N < 1 || d.rows < 1 || d.groups < 1) return 1;
+    const int cols = d.b32 ? R16Shape<true>::kCols : R16Shape<false>::kCols;
+    Rows16Params p = {};
+    p.A = d.A; p.B = nullptr; p.C = d.C; p.R = d.R;
+    p.lda = d.lda; p.sA = 0; p.ldb = d.K; p.sB = 0; p.ldc = d.ldc; p.sC = 0;
+    p.G = 1; p.M = d.rows; p.N = d.N; p.K = d.K; p.shift = d.shift; p.b_shift = 0; p.init = d.init;
+    p.row_tiles = 1;
+    p.col_groups = (d.N + cols - 1) / cols;
+    p.nslices = 1;
+    p.grp_seg = d.seg; p.grp_tiles = d.tiles; p.grp_ntiles = d.ntiles; p.grp_b = d.B;
+    // the grid covers the worst case of the tile table (the host never learns the segment sizes): rows / 32 + groups
+    // tiles of 32 rows, two halves each
+    const long items = ((long)d.rows / 32 + d.groups) * 2 * p.col_groups;
+    return r16_run(d.b32 ? gemm_rows16_kernel<true, true> : gemm_rows16_kernel<false, true>, p, items);
+}
+
+}  // namespace zk

@@ -1,5 +1,5 @@
 // Error channel, stopwatch and the host-side table initialisers of libint64gemm.so.
-#include "common.h"
+#include "gemm.h"
 #include "../../include/int64gemm.h"
 
 #include <cmath>
@@ -89,7 +89,7 @@ void zk_clear_error(void)
 
 size_t zk_workspace_bytes(void)
 {
-    return zk::gemm_mfma_workspace_bytes(nullptr) + zk::act_workspace_bytes();
+    return zk::gemm_mfma_workspace_bytes(nullptr) + zk::gemm_rows16_workspace_bytes() + zk::act_workspace_bytes();
 }
 
 size_t zk_prepared_weights_bytes(void)
@@ -102,6 +102,7 @@ size_t zk_prepared_weights_bytes(void)
 void zk_release_workspace(void)
 {
     zk::gemm_mfma_release_workspace();       // waits for the device first
+    zk::gemm_rows16_release_workspace();
     zk::act_release_workspace();
 }
 
