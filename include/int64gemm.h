@@ -204,7 +204,8 @@ void moe_combine(const int64_t *ye, const int64_t *weights, const int *sorted_po
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
 void zk_gemm_set_path(int path);
 int zk_gemm_get_path(void);
-/* What the last GEMM-like call used: path (1/2) and the limb counts of A and B (0 for the VALU path). */
+/* What the last GEMM-like call used: path (1/2) and the limb counts of A and B (0 for the VALU path, and for the
+ * MFMA kernels for up to 16 rows, which take their digit counts from the data step by step). */
 void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
 /* i8 digit products per int64 multiply-add in the last GEMM-like call (0 for the VALU path).  At most
  * limbs_a * limbs_b; fewer when the stored bits [shift, shift + 64) of the sum lie below the weight of the top

@@ -9,6 +9,7 @@ namespace zk {
 
 static int g_gemm_path = kPathAuto;
 static int g_last_path = 0, g_last_la = 0, g_last_lb = 0;
+static bool g_last_digits = false;      // the last call ran on kernels with fixed digit counts (gemm_mfma.hip), whose plan and planes are reported
 static long g_grouped_mfma_calls = 0;
 
 bool gemm_dispatch(const char *name, const GemmDesc &d)
@@ -20,7 +21,7 @@ bool gemm_dispatch(const char *name, const GemmDesc &d)
     // product.  One row against [18432,7168]: 0.19 -> 0.087 ms; against [576,7168] the stream wins, 9 against 22 us.)
     const bool prepared = g_gemm_path != kPathValu && !d.b32 && (long)d.N * d.K >= (16L << 20) && gemm_mfma_is_prepared(d.B);
     if (g_gemm_path != kPathMfma && !prepared && gemm_gemv_launch(d)) {
-        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
         return check_launch(name);
     }
     // up to 16 rows against k-contiguous weights: the 16-row MFMA tiles, digit counts taken from the data on the device
@@ -28,7 +29,7 @@ bool gemm_dispatch(const char *name, const GemmDesc &d)
     if (g_gemm_path != kPathValu && !gemm_mfma_is_prepared(d.B)) {
         const int rc = gemm_rows16_launch(d);
         if (rc == 0) {
-            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0;
+            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
             return check_launch(name);
         }
         if (rc < 0) return false;
@@ -39,17 +40,17 @@ bool gemm_dispatch(const char *name, const GemmDesc &d)
         // one from running on the other path), -1: failed and recorded
         const int rc = gemm_mfma_launch(d, &la, &lb);
         if (rc == 0) {
-            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb;
+            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb; g_last_digits = true;
             return check_launch(name);
         }
         if (rc < 0) return false;
     }
     if (g_gemm_path != kPathMfma && prepared && gemm_gemv_launch(d)) {
-        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
         return check_launch(name);
     }
     gemm_valu_launch(d);
-    g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+    g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
     return check_launch(name);
 }
 
@@ -66,25 +67,28 @@ void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
     const bool prepared = g_gemm_path != kPathValu && !d.b32 && d.rows > 32 && gemm_mfma_is_prepared((const void *)d.B);
     const bool few_rows = g_gemm_path != kPathMfma && d.rows <= kGroupedGemvMaxRows && d.K > 0;
     if (few_rows && !prepared && gemm_gemv_grouped_launch(d)) {
-        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
         check_launch(name);
         return;
     }
-    if (g_gemm_path != kPathValu && !gemm_mfma_is_prepared((const void *)d.B)) {
-        const int rc = gemm_rows16_grouped(d);
+    if (g_gemm_path != kPathValu && d.K > 0) {
+        int la = 0, lb = 0;
+        const int rc = gemm_mfma_grouped(d, &la, &lb);
         if (rc == 0) {
-            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0;
+            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb; g_last_digits = true;
             g_grouped_mfma_calls++;
             check_launch(name);
             return;
         }
         if (rc < 0) return;
     }
-    if (g_gemm_path != kPathValu && d.K > 0) {
-        int la = 0, lb = 0;
-        const int rc = gemm_mfma_grouped(d, &la, &lb);
+    // operands wider than the 32-row kernels take (or K == 0): the 16-row tiles, which take their digit counts from
+    // the data and recompute on the vector ALU what is wider still.  One launch as well, and no wait.  (On the experts'
+    // usual widths the 32-row kernels stream faster: 4.9 against 2.4 TB/s of int32 weights.)
+    if (g_gemm_path != kPathValu) {
+        const int rc = gemm_rows16_grouped(d);
         if (rc == 0) {
-            g_last_path = kPathMfma; g_last_la = la; g_last_lb = lb;
+            g_last_path = kPathMfma; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
             g_grouped_mfma_calls++;
             check_launch(name);
             return;
@@ -92,7 +96,7 @@ void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
         if (rc < 0) return;
     }
     if (few_rows && prepared && gemm_gemv_grouped_launch(d)) {
-        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0;
+        g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
         check_launch(name);
         return;
     }
@@ -246,11 +250,11 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b)
 }
 
 long zk_gemm_guard_hits(void) { return zk::gemm_mfma_guard_hits(); }
-int zk_gemm_last_pairs(void) { return zk::g_last_path == zk::kPathMfma ? zk::gemm_mfma_last_pairs() : 0; }
+int zk_gemm_last_pairs(void) { return zk::g_last_digits ? zk::gemm_mfma_last_pairs() : 0; }
 
 long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
 
-int zk_gemm_last_prepared(void) { return zk::g_last_path == zk::kPathMfma ? zk::gemm_mfma_last_prepared() : 0; }
+int zk_gemm_last_prepared(void) { return zk::g_last_digits ? zk::gemm_mfma_last_prepared() : 0; }
 int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K) { return zk::gemm_mfma_prepare(B, b32, groups, N, K); }
 void zk_gemm_release_weights(const void *B) { zk::gemm_mfma_release(B); }
 

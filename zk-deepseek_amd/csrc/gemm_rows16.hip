@@ -1,15 +1,15 @@
-// GEMM for a handful of rows (M <= 16 per row tile): weight streams on v_mfma_i32_16x16x64_i8, every wavefront on
-// its own, digit counts taken from the data.
+// GEMM for a handful of rows (M <= 16 per row tile): weight streams on v_mfma_i32_16x16x64_i8, digit counts taken
+// from the data.
 //
 // A product of a few activation rows with a wide weight matrix (the MLA down-projections on a short prompt, the routed
 // experts of a MoE layer with ~8 tokens each) is bound by the one pass over the weights, and the 32-row tiles of the
 // general kernel multiply mostly padding there.  This kernel uses the 16x16x64 i8 MFMA, whose operand fragment is 16
-// bytes of ONE row per lane: lane (i, q) = (lane % 16, lane / 16) holds 16 of the 64 k of a step for row i.  A lane can
-// therefore load its own fragment straight from global memory (eight 16-byte loads for int64, four for int32 weights;
-// the four lanes of a row read 64 contiguous bytes per load), split it into balanced base-256 digits in registers
-// (see gemm_mfma.hip for the digit scheme) and feed the matrix pipe: no LDS, no barrier, no cooperation between
-// wavefronts.  Which k a fragment byte stands for does not matter as long as both operands agree, so the byte order
-// follows the loads.
+// bytes of ONE row per lane: lane (i, q) = (lane % 16, lane / 16) holds 16 of the 64 k of a step for row i.  A lane's
+// fragment is therefore a few 16-byte pieces of its own row (the four lanes of a row read 64 contiguous bytes per
+// load): the raw elements travel from global memory straight into LDS (global_load_lds_dwordx4, no registers held
+// while they are under way), each lane reads back what it loaded, splits it into balanced base-256 digits in
+// registers (see gemm_mfma.hip for the digit scheme) and feeds the matrix pipe.  Which k a fragment byte stands for
+// does not matter as long as both operands agree, so the byte order follows the loads.
 //
 // Nothing is guessed.  Before a step is split, the wavefront ORs the magnitudes of what it loaded and picks the digit
 // counts that step needs (3, 4 or 5 per operand, accumulated in nine int32 diagonals per tile).  A wavefront that
@@ -17,11 +17,13 @@
 // outputs with 128-bit multiply-adds on the vector ALU.  Results are exact for every input, no range travels to the
 // host, and the call never waits.
 //
-// A work item is (batch or expert, 16-row tile, group of 32 columns, slice of K); one wavefront = one workgroup = one
-// item, four wavefronts to a workgroup.  With one slice the wavefront stores C and R itself.  With several (a launch too
-// small to fill the device otherwise), the four wavefronts of a workgroup are four slices of one tile: they add up in
-// LDS, the workgroup leaves its 128-bit sums in a slot of scratch and takes a ticket, and the workgroup that arrives
-// last adds the slots, applies rounding term and shift, stores, and resets the ticket for the next call.
+// A workgroup is four wavefronts on the same 16 rows and the same slice of K, each with its own group of columns.
+// The rows of A are loaded once per workgroup (every wavefront a quarter) into a ring of four steps that all four read;
+// each wavefront has a ring of three steps of its own weights.  What bounds such a stream is the bytes under way:
+// the rings keep about 100 KB of weights per compute unit in flight, at the price of one barrier per step.
+// With one slice of K a wavefront stores C and R itself.  With several (a launch too small to fill the device
+// otherwise) every workgroup leaves its wavefronts' 128-bit sums in slots of scratch and a second, small launch adds
+// the slots, applies rounding term and shift and stores.
 #include "gemm_mfma_kernels.h"
 
 namespace zk {
@@ -34,27 +36,26 @@ struct Rows16Params {
     int G, M, N, K, shift, b_shift;
     int64_t init;
     int row_tiles, col_groups, nslices;
-    unsigned long long *acc;             // split K: per (g, row tile, column group) and workgroup of slices, the workgroup's 128-bit sums
+    unsigned long long *acc;             // split K: per (g, row tile, column group) and slice, the wavefront's 128-bit sums
     // grouped mode: rows of A and C form one segment per group, every group has its own B (see GroupedDesc)
     const int *grp_seg, *grp_tiles, *grp_ntiles;
     const void *const *grp_b;
-    int dbg;
 };
 
 constexpr int kR16Fast = 9;              // diagonals the accumulators hold: digit pairs up to (5, 5)
 constexpr int kR16FoldSteps = 16;        // steps between folds of the accumulators (5 pairs * 64 * 2^14 * 16 < 2^31)
 constexpr int kR16Waves = 4;             // wavefronts per workgroup (one per SIMD: the kernel takes most of the register file)
-constexpr int kR16RingBytes = 32 * 1024; // LDS per wavefront: the ring of steps on their way from HBM
+constexpr int kR16StagesA = 4;           // steps of A the workgroup's shared ring holds (8 KB each)
+constexpr int kR16StagesW = 3;           // steps of weights a wavefront's own ring holds (8 KB each)
 
-// 16-column tiles per wavefront: a step of int32 weights is half the bytes of a step of int64 weights
+// 16-column tiles per wavefront: a step of a wavefront's weights is 8 KB either way
 template <bool B32> struct R16Shape {
     static constexpr int kColTiles = B32 ? 2 : 1;
     static constexpr int kCols = 16 * kColTiles;
     static constexpr int kLoadsPerTile = B32 ? 4 : 8;                       // 16-byte loads per lane and column tile
-    static constexpr int kStageBytes = (8 + kColTiles * kLoadsPerTile) * 1024;   // A's eight loads, then the tiles'
-    static constexpr int kStages = kR16RingBytes / kStageBytes;
-    static_assert(kStages >= 2, "the ring holds at least two steps");
+    static_assert(kColTiles * kLoadsPerTile == 8, "eight loads of weights per lane and step");
 };
+constexpr int kR16LdsBytes = kR16StagesA * 8192 + kR16Waves * kR16StagesW * 8192;
 
 // ---- loads that bypass the registers ------------------------------------------------------------------------
 // global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS: one wave-instruction fills
@@ -218,44 +219,42 @@ template <bool B32, bool GRP>
 __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Params p)
 {
     typedef R16Shape<B32> S;
-    constexpr int CT = S::kColTiles, LPT = S::kLoadsPerTile, LPS = 8 + CT * LPT;     // loads per lane and step
+    constexpr int CT = S::kColTiles, LPT = S::kLoadsPerTile;
+    constexpr int LPS = 2 + 8;                       // loads per lane and step: a quarter of A's eight, the weights' eight
     extern __shared__ __attribute__((aligned(16))) unsigned char r16_smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, q = lane >> 4;
-    unsigned char *ring = r16_smem + wave * kR16RingBytes;
-    const unsigned ring_lds = (unsigned)(uintptr_t)ring;             // LDS byte address of this wavefront's ring
+    unsigned char *ring_a = r16_smem;                                               // [stage][load][lane] 16 bytes
+    unsigned char *ring_w = r16_smem + kR16StagesA * 8192 + wave * (kR16StagesW * 8192);
+    const unsigned ring_a_lds = (unsigned)(uintptr_t)ring_a, ring_w_lds = (unsigned)(uintptr_t)ring_w;   // LDS byte addresses
 
-    // wavefront -> item (batch or 32-row tile half, column group, K slice).  With several slices the slice moves fastest:
-    // the wavefronts of a workgroup are then four slices of one output tile and add up in LDS first.  Otherwise the
-    // column group does: the wavefronts that run side by side share their rows of A.
-    unsigned item = blockIdx.x * kR16Waves + wave;                 // (the host keeps the item count below 2^31)
+    // workgroup -> (batch or 32-row tile half, four column groups, K slice); the wavefronts take the column groups
+    unsigned item = blockIdx.x;                                     // (the host keeps the count below 2^31)
+    const int cg4 = (p.col_groups + kR16Waves - 1) / kR16Waves;
     int slice = 0;
     if (p.nslices > 1) { slice = (int)(item % (unsigned)p.nslices); item /= (unsigned)p.nslices; }
-    const int cg = (int)(item % (unsigned)p.col_groups);
-    item /= (unsigned)p.col_groups;
+    const int cg = (int)(item % (unsigned)cg4) * kR16Waves + wave;
+    item /= (unsigned)cg4;
     int g = 0, m0 = 0, m_lim = p.M;
     const void *b_base = p.B;
     long tile_id = 0;                       // index of (g, row tile, column group) among the launch's output tiles
-    bool live = true;
     if (GRP) {
         // item = (32-row tile of the dispatch table, half): 16 rows each
         const int mt = (int)(item >> 1), half = (int)(item & 1);
-        live = mt < *p.grp_ntiles;
-        if (live) {
-            const int e = p.grp_tiles[2 * mt];
-            m0 = p.grp_tiles[2 * mt + 1] + 16 * half;
-            m_lim = p.grp_seg[e + 1];
-            live = m0 < m_lim;
-            b_base = p.grp_b[e];
-        }
+        if (mt >= *p.grp_ntiles) return;                            // (the same for the whole workgroup)
+        const int e = p.grp_tiles[2 * mt];
+        m0 = p.grp_tiles[2 * mt + 1] + 16 * half;
+        m_lim = p.grp_seg[e + 1];
+        if (m0 >= m_lim) return;
+        b_base = p.grp_b[e];
     } else {
         const int rt = (int)(item % (unsigned)p.row_tiles);
         g = (int)(item / (unsigned)p.row_tiles);
-        live = g < p.G;
         m0 = rt * 16;
         tile_id = ((long)g * p.row_tiles + rt) * p.col_groups + cg;
     }
-    if (!live) return;                      // (only without K slices: no barrier lies ahead)
-    const int n0 = cg * S::kCols;
+    // a wavefront past the last column group still loads its quarter of A and meets the others at the barriers
+    const bool live = cg < p.col_groups;
+    const int n0 = (live ? cg : 0) * S::kCols;
 
     // this lane's rows (clamped: the products of rows past the end land in outputs that are never stored)
     int am = m0 + li;
@@ -273,7 +272,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
 
     const int ksteps = (p.K + 63) / 64;
     const int ks_begin = (int)((long)slice * ksteps / p.nslices), ks_end = (int)((long)(slice + 1) * ksteps / p.nslices);
-    // steps that travel through the ring: whole ones, on 16-byte aligned rows; the others are loaded element by element
+    // steps that travel through the rings: whole ones, on 16-byte aligned rows; the others are loaded element by element
     const int full_end = vec ? (p.K / 64 < ks_end ? p.K / 64 : ks_end) : ks_begin;
 
     v4i acc[CT][kR16Fast];
@@ -294,26 +293,23 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
         }
     };
 
-    // stage `st` of the ring <- step ks: A's eight pieces, then every tile's
-    auto issue = [&](int ks, int st) {
+    // step ks on its way: this wavefront's quarter of A's eight pieces into the shared ring, its weights into its own
+    auto issue = [&](int ks) {
         const int k0 = ks * 64;
-        const unsigned base = ring_lds + st * S::kStageBytes;
+        const unsigned base_a = ring_a_lds + ((ks - ks_begin) % kR16StagesA) * 8192;
+        const unsigned base_w = ring_w_lds + ((ks - ks_begin) % kR16StagesW) * 8192;
 #pragma unroll
-        for (int j = 0; j < 8; j++) if (!(p.dbg & 4) || j < 1) lds_dma16(a_row + k0 + frag_k<B32>(q, 2 * j), base + j * 1024); else lds_dma16(a_row, base + j * 1024);
+        for (int h = 0; h < 2; h++) {
+            // (the piece number depends on the wavefront: every j is compiled, one is taken)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (j == 2 * wave + h) lds_dma16(a_row + k0 + frag_k<B32>(q, 2 * j), base_a + j * 1024);
+        }
 #pragma unroll
         for (int ct = 0; ct < CT; ct++)
 #pragma unroll
-            for (int j = 0; j < LPT; j++) {
-                if (p.dbg & 8) {
-                    // bandwidth experiment: each instruction reads whole 256-byte (int32) / 512-byte runs of a row
-                    const int rows_per = B32 ? 4 : 2, lanes_per = 64 / rows_per;
-                    int n = n0 + 16 * ct + rows_per * j + lane / lanes_per;
-                    n = n < p.N ? n : p.N - 1;
-                    const char *rowp = reinterpret_cast<const char *>(b_base) + ((long)g * p.sB + (long)n * p.ldb) * (B32 ? 4 : 8);
-                    lds_dma16(rowp + (long)k0 * (B32 ? 4 : 8) + (lane % lanes_per) * 16, base + (8 + ct * LPT + j) * 1024);
-                } else
-                lds_dma16(w_row[ct] + (long)(k0 + frag_k<B32>(q, (16 / LPT) * j)) * (B32 ? 4 : 8), base + (8 + ct * LPT + j) * 1024);
-            }
+            for (int j = 0; j < LPT; j++)
+                lds_dma16(w_row[ct] + (long)(k0 + frag_k<B32>(q, (16 / LPT) * j)) * (B32 ? 4 : 8), base_w + (ct * LPT + j) * 1024);
     };
 
     RawFrag<false> fa;
@@ -365,35 +361,37 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
         if (++since_fold == kR16FoldSteps) { fold(); since_fold = 0; }
     };
 
-    // the ring: up to kStages steps under way; a stage is refilled as soon as its step sits in registers
+    // Three steps under way.  In iteration ks: this wavefront's loads of step ks have landed (at most the two steps issued
+    // after it are outstanding); behind the barrier so have everybody's quarters of A, and everybody has read the step
+    // before out of the ring; the step moves into registers; step ks + 3 is issued into the stages that just became free
+    // (its weights into the stage read a moment ago, its rows of A into the stage of step ks - 1).
 #pragma unroll
-    for (int st = 0; st < S::kStages; st++)
-        if (ks_begin + st < full_end && !(p.dbg & 2)) issue(ks_begin + st, st);
-    int st = 0;
-    for (int ks = ks_begin; ks < full_end && !wide; ks++) {
-        // everything issued after step ks: the steps ks+1 .. ks+kStages-1 that exist
-        const int behind = full_end - 1 - ks < S::kStages - 1 ? full_end - 1 - ks : S::kStages - 1;
-        if (behind >= S::kStages - 1) wait_vmcnt<(S::kStages - 1) * LPS>();
-        else if (S::kStages > 2 && behind == S::kStages - 2) wait_vmcnt<(S::kStages > 2 ? S::kStages - 2 : 0) * LPS>();
+    for (int d = 0; d < kR16StagesW; d++)
+        if (ks_begin + d < full_end) issue(ks_begin + d);
+    for (int ks = ks_begin; ks < full_end; ks++) {
+        const int behind = full_end - 1 - ks;
+        if (behind >= 2) wait_vmcnt<2 * LPS>();
+        else if (behind == 1) wait_vmcnt<LPS>();
         else wait_vmcnt<0>();
-        const unsigned char *src = ring + st * S::kStageBytes + lane * 16;
+        __syncthreads();
+        const unsigned char *src_a = ring_a + ((ks - ks_begin) % kR16StagesA) * 8192 + lane * 16;
+        const unsigned char *src_w = ring_w + ((ks - ks_begin) % kR16StagesW) * 8192 + lane * 16;
 #pragma unroll
-        for (int j = 0; j < 8; j++) fa.v[j] = *reinterpret_cast<const v4i *>(src + j * 1024);
+        for (int j = 0; j < 8; j++) fa.v[j] = *reinterpret_cast<const v4i *>(src_a + j * 1024);
 #pragma unroll
         for (int ct = 0; ct < CT; ct++)
 #pragma unroll
-            for (int j = 0; j < LPT; j++) fw[ct].v[j] = *reinterpret_cast<const v4i *>(src + (8 + ct * LPT + j) * 1024);
-        if (ks + S::kStages < full_end) {
-            // (the reads above must have returned before the stage is overwritten)
+            for (int j = 0; j < LPT; j++) fw[ct].v[j] = *reinterpret_cast<const v4i *>(src_w + (ct * LPT + j) * 1024);
+        if (ks + kR16StagesW < full_end) {
+            // (the reads above must have returned before their stage is overwritten)
             __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0)
-            if (!(p.dbg & 2)) issue(ks + S::kStages, st);
+            issue(ks + kR16StagesW);
         }
-        st = st + 1 == S::kStages ? 0 : st + 1;
-        if (!(p.dbg & 1)) process();
+        if (live && !wide) process();
     }
     wait_vmcnt<0>();
-    // steps outside the ring (a partial last step, rows that are not 16-byte aligned): element by element
-    for (int ks = full_end; ks < ks_end && !wide; ks++) {
+    // steps outside the rings (a partial last step, rows that are not 16-byte aligned): element by element
+    for (int ks = full_end; ks < ks_end && live && !wide; ks++) {
         const int k0 = ks * 64, k_left = p.K - k0;
 #pragma unroll
         for (int b = 0; b < 16; b++) {
@@ -417,6 +415,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
             }
         process();
     }
+    if (!live) return;
     fold();
     if (wide) {
         // Values beyond five digits (2^38) somewhere in this item's slice: every lane recomputes its outputs with
@@ -445,50 +444,29 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
         }
     }
 
-    // accumulator register r of lane (li, q) holds row 4*q + r, column li of its 16x16 tile
-    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
-    auto store = [&](int ct, int r, uint64_t lo, uint64_t hi) {
-        const int m = m0 + 4 * q + r, n = n0 + 16 * ct + li;
-        const long o = (long)g * p.sC + (long)m * p.ldc + n;
-        p.C[o] = (int64_t)((lo >> p.shift) | ((hi << 1) << (63 - p.shift)));
-        if (p.R) p.R[o] = (int64_t)(lo & rmask);
-    };
     if (p.nslices == 1) {
+        // accumulator register r of lane (li, q) holds row 4*q + r, column li of its 16x16 tile
+        const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
 #pragma unroll
         for (int ct = 0; ct < CT; ct++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                if (m0 + 4 * q + r >= m_lim || n0 + 16 * ct + li >= p.N) continue;
+                const int m = m0 + 4 * q + r, n = n0 + 16 * ct + li;
+                if (m >= m_lim || n >= p.N) continue;
                 const u128 s = sums[ct][r] + (u128)(i128)p.init;
-                store(ct, r, (uint64_t)s, (uint64_t)(s >> 64));
+                const uint64_t lo = (uint64_t)s, hi = (uint64_t)(s >> 64);
+                const long o = (long)g * p.sC + (long)m * p.ldc + n;
+                p.C[o] = (int64_t)((lo >> p.shift) | ((hi << 1) << (63 - p.shift)));
+                if (p.R) p.R[o] = (int64_t)(lo & rmask);
             }
         return;
     }
-    // Several slices.  The four wavefronts of the workgroup hold four slices of one tile: they meet in LDS (the rings are
-    // idle by now), the first one adds the workgroup's sums into the tile's zeroed scratch and counts in, and the
-    // workgroup that arrives last finishes the tile.
-    u128 *meet = reinterpret_cast<u128 *>(r16_smem);              // [wave][output][lane]
-    if (p.dbg & 64) return;
-    __syncthreads();
-#pragma unroll
-    for (int ct = 0; ct < CT; ct++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) meet[(wave * (CT * 4) + ct * 4 + r) * 64 + lane] = sums[ct][r];
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int ct = 0; ct < CT; ct++)
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int w = 1; w < kR16Waves; w++) sums[ct][r] += meet[(w * (CT * 4) + ct * 4 + r) * 64 + lane];
-    // the workgroup's sums go to its own slot of the tile's scratch; a second launch adds the slots up
+    // Several slices: the sums go to this slice's slot of the tile's scratch, and a second launch adds the slots up.
     // (Finishing inside this kernel was measured first.  Adding into one slot with atomics: fourteen workgroups adding 512
     // sums each spent 3.4 us in dependent round trips to the memory side, and every further slice 0.3 us.  A ticket with
     // the last arriver adding the slots: a round trip for the stores, one for the ticket, and several for the loads,
     // since nothing that crosses the dies may be fenced or cached.  A launch boundary costs less than either.)
-    const int groups = p.nslices / kR16Waves, grp = slice / kR16Waves;
-    u128 *slot = reinterpret_cast<u128 *>(p.acc) + ((long)tile_id * groups + grp) * (CT * 4 * 64);
+    u128 *slot = reinterpret_cast<u128 *>(p.acc) + ((long)tile_id * p.nslices + slice) * (CT * 4 * 64);
 #pragma unroll
     for (int ct = 0; ct < CT; ct++)
 #pragma unroll
@@ -510,7 +488,7 @@ __global__ __launch_bounds__(256) void gemm_rows16_finish_kernel(Rows16Params p)
     const int rt = (int)(t2 % p.row_tiles), g = (int)(t2 / p.row_tiles);
     const int m = rt * 16 + 4 * (lane >> 4) + r, n = cg * R16Shape<B32>::kCols + 16 * ct + (lane & 15);
     if (m >= p.M || n >= p.N) return;
-    const int groups = p.nslices / kR16Waves;
+    const int groups = p.nslices;
     const u128 *slot = reinterpret_cast<const u128 *>(p.acc) + tile_id * groups * PER + o;
     u128 s = (u128)(i128)p.init;
 #pragma unroll 8
@@ -526,8 +504,8 @@ __global__ __launch_bounds__(256) void gemm_rows16_finish_kernel(Rows16Params p)
 namespace zk {
 
 // ---- host side ---------------------------------------------------------------------------------------------
-// Scratch of the split-K launches, kept between calls: slots of 8 KB (the 128-bit sums of one workgroup for one output
-// tile).  Every slot a launch reads has been written by that launch: nothing needs clearing.
+// Scratch of the split-K launches, kept between calls: slots of 8 KB (the 128-bit sums of one wavefront: one output tile,
+// one slice of K).  Every slot a launch reads has been written by that launch: nothing needs clearing.
 static unsigned long long *g_r16_acc = nullptr;
 static size_t g_r16_slots = 0;
 static int g_r16_cus = 0;
@@ -570,19 +548,17 @@ static int r16_scratch(size_t slots)
     return 0;
 }
 
-// How many slices of K per output tile.  One workgroup (four wavefronts) fits a compute unit, so a launch runs in
-// rounds of `cus` workgroups; the slices are a multiple of four (a workgroup's wavefronts add up in LDS before they touch
-// the scratch) and the count that minimises rounds x steps per wavefront wins, a split being charged the second launch.
-static int r16_slices(long tiles, int K, int cus)
+// How many slices of K.  One workgroup fits a compute unit, so a launch runs in rounds of `cus` workgroups; the count
+// that minimises rounds x steps per wavefront wins, a split being charged the second launch.
+static int r16_slices(long wg_tiles, int K, int cus)
 {
     const int ksteps = (K + 63) / 64;
     // in units of one step of one wavefront (about a microsecond): start-up of a round, the finishing launch
     const double round_cost = 3.0, finish_cost = 4.0;
     int best = 1;
     double best_cost = 0;
-    for (int n = 1; n <= ksteps / 2 || n == 1; n = n == 1 ? kR16Waves : n + kR16Waves) {
-        const long wgs = (tiles * n + kR16Waves - 1) / kR16Waves;
-        const long rounds = (wgs + cus - 1) / cus;
+    for (int n = 1; n == 1 || n <= ksteps / 2; n++) {
+        const long rounds = (wg_tiles * n + cus - 1) / cus;
         const double cost = rounds * ((double)((ksteps + n - 1) / n) + round_cost) + (n > 1 ? finish_cost : 0.0);
         if (n == 1 || cost < best_cost) { best = n; best_cost = cost; }
     }
@@ -605,17 +581,15 @@ static bool r16_fill(const GemmDesc &d, Rows16Params &p)
     p.row_tiles = (d.M + 15) / 16;
     p.col_groups = (d.N + cols - 1) / cols;
     p.nslices = 1;
-    p.dbg = getenv("ZK_R16_DBG") ? atoi(getenv("ZK_R16_DBG")) : 0;
     return true;
 }
 
 typedef void (*Rows16Kernel)(Rows16Params);
 
-static int r16_run(Rows16Kernel fn, const Rows16Params &p, long items)
+static int r16_run(Rows16Kernel fn, const Rows16Params &p, long blocks)
 {
-    const long blocks = (items + kR16Waves - 1) / kR16Waves;
-    if (items > 0x7FFFFFF0L) return 1;
-    constexpr int lds = kR16Waves * kR16RingBytes;
+    if (blocks > 0x7FFFFFF0L) return 1;
+    constexpr int lds = kR16LdsBytes;
     static const void *raised[4] = {};
     bool seen = false;
     for (const void *f : raised) seen = seen || f == (const void *)fn;
@@ -638,19 +612,23 @@ int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_sl
     Rows16Params p;
     if (!r16_fill(d, p)) return 1;
     const long tiles = (long)d.G * p.row_tiles * p.col_groups;
+    const long wg_tiles = (long)d.G * p.row_tiles * ((p.col_groups + kR16Waves - 1) / kR16Waves);
     if (tiles > (1L << 24)) return 1;
-    const int slices = r16_slices(tiles, d.K, r16_cus());
+    const int slices = r16_slices(wg_tiles, d.K, r16_cus());
     if (slices > 1) {
-        const size_t slots = (size_t)tiles * (slices / kR16Waves);
+        const size_t slots = (size_t)tiles * slices;
         if (acc) {
-            if (slots <= max_slots) { p.acc = acc; p.nslices = slices; }
+            // a caller's scratch: as many slices as its slots hold
+            const long fit = (long)(max_slots / (size_t)tiles);
+            const int use = slices < fit ? slices : (int)fit;
+            if (use > 1) { p.acc = acc; p.nslices = use; }
         } else {
             const int rc = r16_scratch(slots);
             if (rc < 0) return -1;
             if (rc == 0) { p.acc = g_r16_acc; p.nslices = slices; }
         }
     }
-    const int rc = r16_run(d.b32 ? gemm_rows16_kernel<true, false> : gemm_rows16_kernel<false, false>, p, tiles * p.nslices);
+    const int rc = r16_run(d.b32 ? gemm_rows16_kernel<true, false> : gemm_rows16_kernel<false, false>, p, wg_tiles * p.nslices);
     if (rc != 0 || p.nslices == 1) return rc;
     const long threads = tiles * (d.b32 ? R16Shape<true>::kColTiles : R16Shape<false>::kColTiles) * 4 * 64;
     const dim3 grid((unsigned)((threads + 255) / 256));
@@ -674,8 +652,8 @@ int gemm_rows16_grouped(const GroupedDesc &d)
     p.grp_seg = d.seg; p.grp_tiles = d.tiles; p.grp_ntiles = d.ntiles; p.grp_b = d.B;
     // the grid covers the worst case of the tile table (the host never learns the segment sizes): rows / 32 + groups
     // tiles of 32 rows, two halves each
-    const long items = ((long)d.rows / 32 + d.groups) * 2 * p.col_groups;
-    return r16_run(d.b32 ? gemm_rows16_kernel<true, true> : gemm_rows16_kernel<false, true>, p, items);
+    const long blocks = ((long)d.rows / 32 + d.groups) * 2 * ((p.col_groups + kR16Waves - 1) / kR16Waves);
+    return r16_run(d.b32 ? gemm_rows16_kernel<true, true> : gemm_rows16_kernel<false, true>, p, blocks);
 }
 
 }  // namespace zk
