@@ -200,6 +200,17 @@ void int64_grouped_bmm_launcher(const int64_t *A, const void *const *B_ptrs, int
                                 int rows, int K, int N);
 void moe_combine(const int64_t *ye, const int64_t *weights, const int *sorted_pos, int64_t *y, int T, int K, int N, int shift);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the product of int64_64/32_bmm_broadcast_launcher (b32 != 0: B
+ * holds int32) for up to 16 rows, a_rescale fixed at 1 and b_rescale a positive power of two, on kernels whose scratch
+ * (the partial sums of a K split) is a static 8 MB array in device memory instead of a buffer the library allocates.
+ * It allocates nothing, frees nothing and waits for nothing.  Limits: M <= 16 and Bdim * M * N <= 2^20 outputs; anything
+ * beyond is rejected with error 3.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, two threads) race.  Nothing in the array needs clearing: a call writes every slot it reads.  Same bits as the
+ * existing entry points; R may be NULL. */
+void int64_bmm_broadcast_noalloc(const int64_t *A, const void *B, int b32, int64_t *C, int64_t *R,
+                                 int64_t b_rescale, int64_t c_rescale, int Bdim, int M, int K, int N);
+
 /* GEMM instruction path for the bmm launchers and the einsums: 0 = automatic (default),
  * 1 = native VALU 64-bit multiply-add chains, 2 = limb-decomposed i8 MFMA.  Results are identical. */
 void zk_gemm_set_path(int path);

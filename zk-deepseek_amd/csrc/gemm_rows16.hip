@@ -511,6 +511,8 @@ static size_t g_r16_slots = 0;
 static int g_r16_cus = 0;
 
 constexpr size_t kR16SlotBytes = 8 * 64 * 16;
+constexpr int kNoAllocMaxRows = 16;                        // limits of int64_bmm_broadcast_noalloc
+constexpr long kNoAllocMaxOutputs = 1L << 20;
 
 size_t gemm_rows16_workspace_bytes() { return g_r16_slots * kR16SlotBytes; }
 
@@ -657,3 +659,69 @@ int gemm_rows16_grouped(const GroupedDesc &d)
 }
 
 }  // namespace zk
+
+// ---- the entry point that allocates nothing -----------------------------------------------------------------
+// Callers under HIP graph capture, tight serving loops and harnesses that forbid it cannot call hipMalloc.  For them the
+// scratch of the split-K launches is a file-scope device array: each GPU the library runs on holds its own copy, at its
+// own address, until the process ends.  The array's name is a host-side stand-in, not a device address: its address on
+// the current device is looked up once per device and that pointer is what the kernels get.
+namespace zk {
+
+constexpr size_t kNoAllocSlots = 1024;                                     // 8 MB: slots of 8 KB
+static __device__ __align__(256) unsigned char scratch[kNoAllocSlots * kR16SlotBytes];
+
+constexpr int kNoAllocMaxDevices = 64;
+static unsigned long long *g_noalloc_ptr[kNoAllocMaxDevices] = {};
+
+// the scratch array's address on the current device (null and an error recorded if it cannot be had)
+static unsigned long long *noalloc_scratch(const char *name)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kNoAllocMaxDevices) {
+        set_error(kLaunchFailure, "%s: cannot tell the current device", name);
+        return nullptr;
+    }
+    if (!g_noalloc_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            set_error(kLaunchFailure, "%s: cannot find the scratch array on device %d", name, dev);
+            return nullptr;
+        }
+        g_noalloc_ptr[dev] = reinterpret_cast<unsigned long long *>(ptr);
+    }
+    return g_noalloc_ptr[dev];
+}
+
+}  // namespace zk
+
+extern "C" void int64_bmm_broadcast_noalloc(const int64_t *A, const void *B, int b32, int64_t *C, int64_t *R,
+                                            int64_t b_rescale, int64_t c_rescale, int Bdim, int M, int K, int N)
+{
+    const char *name = "int64_bmm_broadcast_noalloc";
+    using namespace zk;
+    if (Bdim < 0 || M < 0 || K < 0 || N < 0) { set_error(kBadArgument, "%s: negative dimension", name); return; }
+    if (c_rescale < 0 || c_rescale > 63) { set_error(kBadArgument, "%s: shift %lld outside [0,63]", name, (long long)c_rescale); return; }
+    if (b_rescale <= 0 || (b_rescale & (b_rescale - 1)) != 0) {
+        set_error(kBadArgument, "%s: the divisor of B must be a positive power of two", name);
+        return;
+    }
+    if (M > kNoAllocMaxRows) { set_error(kUnsupportedSize, "%s: %d rows, at most %d", name, M, kNoAllocMaxRows); return; }
+    if ((long)Bdim * M * N > kNoAllocMaxOutputs) {
+        set_error(kUnsupportedSize, "%s: %ld outputs, at most %ld", name, (long)Bdim * M * N, kNoAllocMaxOutputs);
+        return;
+    }
+    if ((long)Bdim * M * N == 0) return;
+    if (!A || !B || !C) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    unsigned long long *ptr = noalloc_scratch(name);
+    if (!ptr) return;
+    GemmDesc d;
+    d.A = A; d.lda = K; d.sA = (long)M * K;
+    d.B = B; d.b32 = b32 ? 1 : 0; d.ldbn = K; d.ldbk = 1; d.sB = 0;
+    d.C = C; d.R = R; d.ldc = N; d.sC = (long)M * N;
+    d.G = Bdim; d.M = M; d.N = N; d.K = K;
+    d.shift = (int)c_rescale; d.init = 0; d.a_rs = 1; d.b_rs = b_rescale;
+    // (a K split that would need more slots than the array has is cut down to what fits; one slice needs none)
+    if (gemm_rows16_launch(d, ptr, kNoAllocSlots) == 1) set_error(kUnsupportedSize, "%s: shape outside what the 16-row kernels take", name);
+}
+
