@@ -1,5 +1,7 @@
 """Parity of the HIP library against the CPU oracle, bit for bit, through the C ABI (via the `kernel`
 module, whose functions only allocate outputs and pass device pointers).  Needs an MI355X."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -7,6 +9,11 @@ import torch
 from util import rand_i32, rand_i64
 
 pytestmark = pytest.mark.gpu
+
+# ZK_TEST_SEEDS=n multiplies the seed ranges of the three randomly drawn problem sets below (40, 20 and 10 seeds by
+# default), e.g. `ZK_TEST_SEEDS=200 python -m pytest tests/test_gpu_parity.py -m gpu -x -q -k seeded_random` runs 8000 +
+# 4000 + 2000 seeds and stops at the first mismatch
+SEEDS = max(1, int(os.environ.get("ZK_TEST_SEEDS", "1") or 1))
 
 
 @pytest.fixture(scope="module")
@@ -426,7 +433,7 @@ def test_gemm_config4_full_size_sampled(K, oracle, path, full_range):
     assert torch.equal(C1, torch.roll(C0, 1, dims=1))
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(40 * SEEDS))
 def test_gemm_seeded_random_problems(K, oracle, seed):
     """a sweep no hand-picked list would make: random batch, shape, operand widths, weight type and shift per case, on
     the MFMA path (whole tiles, edge tiles, 32-row tiles, K split, digit planes or not, few or many diagonals kept)"""
@@ -451,7 +458,7 @@ def test_gemm_seeded_random_problems(K, oracle, seed):
     K.lib.zk_gemm_set_path(0)
 
 
-@pytest.mark.parametrize("seed", range(20))
+@pytest.mark.parametrize("seed", range(20 * SEEDS))
 def test_einsums_seeded_random_problems(K, oracle, seed):
     """the four einsums on random shapes and operand widths (strided A rows, k-major and int32 B, per-head batches)"""
     rng = np.random.default_rng(9500 + seed)
@@ -1252,7 +1259,7 @@ def test_bf16_checkpoint_quantisation(K, oracle):
     K.lib.zk_clear_error()
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(10 * SEEDS))
 def test_rowwise_kernels_seeded_random_problems(K, oracle, seed):
     """softmax, activations and RMSNorm on random row lengths, row counts, magnitudes and weight types"""
     rng = np.random.default_rng(9800 + seed)

@@ -246,11 +246,12 @@ def test_softmax_q19_uniform_row_and_mask(oracle):
 
 def test_softmax_q19_single_element_steps(oracle):
     """hand-computed from the definition: d=2^19 (x = max - 1.0): y = 756388, k = 1, f = 232100, LUT[113] >> 1."""
-    lut = oracle.softmax_init_q19()
     x = np.array([0, -(1 << 19)], np.int64).reshape(1, 1, 1, 2)
-    _, w = oracle.softmax_q19(x)
-    y = 756388
-    assert w[0, 0, 0, 1] == lut[(y & 0x7FFFF) >> 11] >> (y >> 19)
+    C, w = oracle.softmax_q19(x)
+    # worked by hand from inference/int64_gemm.cu:700-708 and the table the circuits hold (zk/src/index.ts:2645-2681):
+    # y = (2^19 * 756388) >> 19 = 756388, k = 1, f = 232100, index 113, entry 386095, w = 386095 >> 1
+    assert w[0, 0, 0].tolist() == [524288, 193047]
+    assert C[0, 0, 0].tolist() == [383193, 141094]          # floor(w * 2^19 / (524288 + 193047))
     assert abs(w[0, 0, 0, 1] / 2 ** 19 - math.exp(-1)) < 2e-3
 
 
@@ -280,16 +281,16 @@ def test_sigmoid_silu_special_values_and_float(oracle, Q):
 
 def test_sigmoid_q23_hand_steps(oracle):
     """x = -1.0: y = (2^23 * 12102203) >> 23 = 12102203; k = 1, f = 3713595, t = LUT[113]; u = t << 1."""
-    lut = oracle.silu_init_q23()
+    # literals worked by hand from inference/int64_gemm.cu:932-945 with the table the circuits hold
+    # (zk/src/index.ts:3382-3418): index 113, entry 11391119, u = 22782238, 2^46 // (2^23 + u)
     x = np.array([-(1 << 23)], np.int64)
-    y = 12102203
-    u = int(lut[(y & 0x7FFFFF) >> 15]) << (y >> 23)
-    assert oracle.sigmoid_q23(x)[0] == (1 << 46) // ((1 << 23) + u)
+    assert oracle.sigmoid_q23(x)[0] == 2257517
+    assert oracle.silu_q23(x)[0] == (-(1 << 23) * 2257517) >> 23 == -2257517
     # q23 negates before the shift, q25 after: they differ in rounding for positive inputs
+    # x = 3, q23: y = (-3 * 12102203) >> 23 = -5, k = -1, f = 2^23 - 5, index 255; q25: y = -((3 * 48408813) >> 25) = -4
     x = np.array([3], np.int64)
-    assert oracle.sigmoid_q23(x)[0] == (1 << 46) // ((1 << 23) + (int(lut[255]) >> 1))    # y = -5 -> k=-1, f=2^23-5
-    lut25 = oracle.silu_init_q25()
-    assert oracle.sigmoid_q25(x)[0] == (1 << 50) // ((1 << 25) + (int(lut25[255]) >> 1))   # y = -(4) -> k=-1
+    assert oracle.sigmoid_q23(x)[0] == 4199982
+    assert oracle.sigmoid_q25(x)[0] == 16799929
 
 
 # -------------------------------------------------------------------- float -> fixed converters ---
@@ -424,3 +425,87 @@ def test_gate_route_hand_case_and_ties(oracle):
     # without a bias a group is scored by its maximum: 10, 7, 9, 7 -> groups 0 and 2
     w, idx, raw = oracle.gate_route(scores, None, 4, 2, 3)
     assert idx.tolist() == [[0, 4, 5]]
+
+
+# ------------------------------------------------ the proving circuits' own restatement of the kernels ---
+# zk/src/index.ts re-derives every kernel result inside the circuits: a proof only verifies if the witness the kernels
+# wrote satisfies THESE formulas.  They are restated below in Python big integers, following the TypeScript (not the
+# CUDA source the oracle follows), with the tables the circuits hold, and compared with the oracle on random inputs in
+# the model's domain.
+def ts_shr_var(x, k):
+    """shrVar, zk/src/index.ts:2690-2706 / 3425-3440: a shift by the low six bits of k"""
+    return x >> (k & 63)
+
+
+def ts_softmax_row_q19(xs, table, log2e):
+    """calcSumW (zk/src/index.ts:3058-3093) for the sum, the section circuit (:2721-2757) for the quotients"""
+    xmax = max(xs)
+    ws = []
+    for x in xs:
+        d = xmax - x
+        if d > (64 << 19):                      # :3071 (the circuit has no such test: k >= 64 zeroes the same elements)
+            ws.append(0)
+            continue
+        y = (d * log2e) >> 19                   # :3075, :2733
+        k = y >> 19
+        if k >= 64:                             # :3078, :2740
+            ws.append(0)
+            continue
+        f = (y - k * (1 << 19)) >> (19 - 8)     # :3082, :2735
+        ws.append(ts_shr_var(table[f], k))
+    total = sum(ws)
+    return ws, [0 if total == 0 else (w << 19) // total for w in ws]        # :2752-2753
+
+
+def ts_sigmoid_q23(x, table, log2e):
+    """the witness and the constraints of the sigmoid circuit, zk/src/index.ts:3511-3557"""
+    pdt = -x * log2e                            # :3511
+    q = pdt >> 23                               # :3519
+    k = q >> 23                                 # :3521
+    f = q & ((1 << 23) - 1)
+    t = table[f >> (23 - 8)]                    # :3523-3525
+    u = t >> (-k & 63) if k < 0 else (t << (k & 63)) & ((1 << 64) - 1)      # :3551 with shrVar / shlVar on UInt64
+    if abs(k) >= 63:                            # :3553 (`Bool && Bool` in JavaScript yields its second operand)
+        u = 0
+    return (1 << 46) // ((1 << 23) + u)         # :3555
+
+
+def test_softmax_q19_equals_the_circuits_restatement(oracle, zk_tables):
+    table, log2e = zk_tables["q19Table"], zk_tables["LOG2E_Q19"]
+    rng = np.random.default_rng(2721)
+    rows = 0
+    for T, n in ((1, 3000), (2, 2500), (3, 2000), (7, 1500), (31, 800), (64, 500), (128, 300), (200, 200)):
+        x = rng.integers(-(12 << 19), 12 << 19, size=(1, 1, n, T), dtype=np.int64)
+        if T > 1:
+            # causal rows: a masked tail at -2^42 (inference/model.py:1555), and distances right at the clip
+            for r in range(0, n, 3):
+                x[0, 0, r, rng.integers(1, T):] = -(1 << 42)
+            edge = rng.integers(0, n, size=n // 4)
+            x[0, 0, edge, 0] = x[0, 0, edge].max(axis=1) - (1 << 25) - rng.integers(-2, 3, size=edge.size)
+            x[0, 0, edge[::2], T - 1] = x[0, 0, edge[::2]].max(axis=1) - rng.integers(0, 1 << 25, size=edge[::2].size)
+        C, W = oracle.softmax_q19(x)
+        for r in range(n):
+            ws, cs = ts_softmax_row_q19([int(v) for v in x[0, 0, r]], table, log2e)
+            assert W[0, 0, r].tolist() == ws and C[0, 0, r].tolist() == cs, (T, r)
+        rows += n
+    assert rows >= 10000
+
+
+def test_sigmoid_silu_q23_equal_the_circuits_restatement(oracle, zk_tables):
+    """the quotient q = 2^46 // (2^23 + u) as the circuits constrain it, for k on both sides of 0, |x| up to the kernel's
+    saturation limit on the positive side and down to -27.7 (beyond it `t << k` leaves 64 bits: hardware-defined in the
+    CUDA build, parity unpinned).  SiLU is (x * q) >> 23 with that q (inference/int64_gemm.cu:945); the circuits write
+    x.mul(q).div(2^23) (:3651), whose rounding for negative x is o1js's and is not pinned here."""
+    table, log2e = zk_tables["q23Table"], zk_tables["LOG2E_Q23"]
+    rng = np.random.default_rng(3511)
+    one = 1 << 23
+    x = np.concatenate([rng.integers(-27 * one, 64 * one, size=20000, dtype=np.int64),
+                        rng.integers(-one, one, size=6000, dtype=np.int64),           # k = -1, 0 and 1
+                        rng.integers(-64, 64, size=200, dtype=np.int64),
+                        np.array([0, 1, -1, 64 * one - 1, 43 * one, 44 * one, -27 * one], np.int64)])
+    sig, silu = oracle.sigmoid_q23(x), oracle.silu_q23(x)
+    for i, v in enumerate(x.tolist()):
+        q = ts_sigmoid_q23(v, table, log2e)
+        assert sig[i] == q, v
+        assert silu[i] == (v * q) >> 23, v
+
