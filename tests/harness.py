@@ -32,6 +32,33 @@ class CpuBackend:
     def rmsnorm(self, x2d, w, dim):
         return self.o.RMS_Norm_int64(x2d, w, 1, dim)[0]
 
+    def rmsnorm_with_statistic(self, x2d, w, dim):
+        """(C, the 500-row statistic buffer the reference returns whole: inference/kernel.py:525, 550)"""
+        C, r = self.o.RMS_Norm_int64(x2d, w, 1, dim)
+        if not hasattr(self, "rms500"):
+            self.rms500 = np.zeros((500,), np.int64)
+        self.rms500[:r.shape[0]] = r
+        return C, self.rms500
+
+    # ---- witness dump (inference/model.py:94-102: raw C-order bytes); off unless `out` names a directory
+    out = None
+
+    def save(self, name, t):
+        if self.out is None:
+            return
+        import os
+        path = os.path.join(self.out, name)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "wb") as f:
+            f.write(np.ascontiguousarray(self.to_host(t)).tobytes(order="C"))
+
+    def flush(self):
+        pass
+
+    def weight_bits(self, w):
+        """int32 weights are dumped as their uint32 view (model.py:779): the same bytes"""
+        return w
+
     def residual_rmsnorm(self, x2d, y2d, k, w, dim):
         """(x + y * 2^k, its norm): inference/model.py:1465-1468 op by op"""
         x2d = x2d + y2d * (1 << k)
@@ -46,6 +73,11 @@ class CpuBackend:
 
     def silu_mul(self, r1, r2):
         return (self.silu(r1) * r2) >> 23        # model.py:1048 uses // 2^23, :1280 uses >> 23: the same floor
+
+    def silu_mul_keep(self, r1, r2):
+        """(SiLU values, gate product): the reference dumps the former (model.py:1042, 1274)"""
+        s1 = self.silu(r1)
+        return s1, (s1 * r2) >> 23
 
     def rope(self, x, table):
         return self.o.complex_int64_mul_broadcast(x, table)
@@ -101,9 +133,33 @@ class GpuBackend:
     def rmsnorm(self, x2d, w, dim):
         return self.k.RMS_Norm_int64(x2d.contiguous(), w, 1, dim)[0]
 
+    def rmsnorm_with_statistic(self, x2d, w, dim):
+        return self.k.RMS_Norm_int64(x2d.contiguous(), w, 1, dim)          # (C, the 500-row host buffer)
+
     softmax_scores = CpuBackend.softmax_scores   # the same op-by-op chain, on torch tensors
     silu_mul = CpuBackend.silu_mul
+    silu_mul_keep = CpuBackend.silu_mul_keep
     residual_rmsnorm = CpuBackend.residual_rmsnorm
+    out = None
+
+    def save(self, name, t):
+        """the reference's saveTensor as the reference calls it: a synchronous copy to the host, then the file"""
+        if self.out is None:
+            return
+        import os
+        path = os.path.join(self.out, name)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        if isinstance(t, np.ndarray):
+            t = self.t.from_numpy(np.ascontiguousarray(t))
+        t = t.detach().cpu().contiguous()
+        with open(path, "wb") as f:
+            f.write(t.numpy().tobytes(order="C"))
+
+    def flush(self):
+        pass
+
+    def weight_bits(self, w):
+        return w
 
     def rope(self, x, table):
         return self.k.complex_int64_mul_broadcast(x.contiguous(), table.contiguous())
@@ -141,14 +197,39 @@ class FusedGpuBackend(GpuBackend):
         self.k.silu_mul_q23(r1.contiguous(), r2.contiguous(), out)
         return out
 
+    def silu_mul_keep(self, r1, r2):
+        s1, out = self.t.empty_like(r1), self.t.empty_like(r1)
+        self.k.silu_mul_q23(r1.contiguous(), r2.contiguous(), out, S=s1)
+        return s1, out
+
     def residual_rmsnorm(self, x2d, y2d, k, w, dim):
         xn, c, _ = self.k.RMS_Norm_residual_int64(x2d.contiguous(), y2d.contiguous(), k, w, 1, dim)
         return xn, c
 
+    def rmsnorm_with_statistic(self, x2d, w, dim):
+        # the statistic stays on the device (no wait); the dump writer copies it behind the kernels
+        return self.k.RMS_Norm_int64(x2d.contiguous(), w, 1, dim, host_rms=False)
+
+    def save(self, name, t):
+        """through the library's dump writer: device tensors are handed over as they are (no .cpu())"""
+        if self.out is None:
+            return
+        import os
+        path = os.path.join(self.out, name)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        if isinstance(t, np.ndarray):
+            t = self.t.from_numpy(np.ascontiguousarray(t))
+        self.k.saveTensor(path, t)
+
+    def flush(self):
+        self.k.dump_flush()
+
     def route(self, scores, bias_host, cfg):
         bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
-        w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"])
+        raw = self.t.empty((scores.shape[0], cfg["topk"]), dtype=self.t.int64, device="cuda")
+        w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"], raw_weights=raw)
         self.last_route = (w, idx)
+        self.last_raw_weights = raw
         return w.cpu().numpy(), idx.cpu().numpy()
 
     def routed_experts(self, x, P, cfg):
@@ -160,7 +241,11 @@ class FusedGpuBackend(GpuBackend):
             self._tables_for = key
         t1, t3, t2 = self._tables
         b32 = P["w1"][0].dtype == self.t.int32
-        return self.k.moe_experts(x[0].contiguous(), w, idx, t1, t3, t2, b32, cfg["inter"], cfg["c13"], cfg["c2"])
+        dump = None
+        if self.out is not None and getattr(self, "layer_dir", None):
+            import os
+            dump = os.path.join(self.out, self.layer_dir)
+        return self.k.moe_experts(x[0].contiguous(), w, idx, t1, t3, t2, b32, cfg["inter"], cfg["c13"], cfg["c2"], dump_dir=dump)
 
 
 class CheckedGpuBackend(GpuBackend):
@@ -226,6 +311,9 @@ class CheckedGpuBackend(GpuBackend):
         self._count("rmsnorm", want.size)
         return out
 
+    def rmsnorm_with_statistic(self, x2d, w, dim):
+        return self.rmsnorm(x2d, w, dim), self.k.rms
+
     def rope(self, x, table):
         out = super().rope(x, table)
         want = self.cpu.rope(np.ascontiguousarray(x.cpu().numpy()), np.ascontiguousarray(table.cpu().numpy()))
@@ -249,52 +337,86 @@ class CheckedGpuBackend(GpuBackend):
         return out
 
 
-def expert_ffn(be, x, w1, w2, w3, c13, c2):
+def expert_ffn(be, x, w1, w2, w3, c13, c2, dump=None):
     """gate/up GEMMs, SiLU gate, down GEMM: MLP_int.forward / Expert_int.forward
     (inference/model.py:1018-1049, 1247-1281).  x [1,M,dim] Q23 activations."""
     r1, _ = be.linear(x, w1, c13)
     r2, _ = be.linear(x, w3, c13)
-    h = be.silu_mul(r1, r2)
+    if dump:                                  # file names of model.py:1037-1042 (shared expert) / :1269-1274 (routed)
+        s1, h = be.silu_mul_keep(r1, r2)
+        be.save(dump + "_x.bin", r1)
+        be.save(dump + "_y.bin", s1)
+    else:
+        h = be.silu_mul(r1, r2)
     y, _ = be.linear(h, w2, c2)
     return y
 
 
-def attention_scores_softmax_pv(be, q_nope, q_pe, kv_cache, pe_cache, causal=True):
+def attention_scores_softmax_pv(be, q_nope, q_pe, kv_cache, pe_cache, causal=True, layer_dir=None):
     """scores = ((q_nope.kv + 11)>>23 + (q_pe.pe + 10)>>21) * 94 // 695 + mask; softmax_q19; P.V >> 23
     (inference/model.py:884-936).  q_nope [1,S,H,C], q_pe [1,S,H,R], kv_cache [1,T,C], pe_cache [1,T,R]."""
     s1 = be.einsum("einsum_bshc_btc_bsht", q_nope, kv_cache, 23)
     s2 = be.einsum("einsum_bshc_btc_bsht", q_pe, pe_cache, 21)
     scores, p = be.softmax_scores(s1, s2, be.causal_mask(s1.shape[1], s1.shape[3]) if causal else None)
+    if layer_dir:
+        be.save(layer_dir + "/scores_softmax_x.bin", scores)            # model.py:913, 918
+        be.save(layer_dir + "/scores_softmax_y.bin", p)
     out = be.einsum("einsum_bsht_btc_bshc", p, kv_cache, 23)
     return scores, p, out
 
 
-def mla(be, x, P, freqs, cfg):
+def mla(be, x, P, freqs, cfg, layer_dir=None):
     """MLA.forward in absorb mode at start_pos = 0 (inference/model.py:747-957).  x [1,S,dim]."""
     S, H = x.shape[1], cfg["heads"]
     cq, ckv = cfg.get("c_q", 30), cfg.get("c_kv", 29)           # the model's scales (model.py:772-833); tests may pick others
-    q_down, _ = be.linear(x, P["wq_a"], cq)
-    q_normed = be.rmsnorm(q_down[0], P["q_norm"], cfg["q_lora"])[None]
+    q_down, q_down_rem = be.linear(x, P["wq_a"], cq)
+    q_normed, q_rms = be.rmsnorm_with_statistic(q_down[0], P["q_norm"], cfg["q_lora"])
+    q_normed = q_normed[None]
+    if layer_dir:                             # model.py:776-793
+        be.save(layer_dir + "/wq_a_x.bin", x)
+        be.save(layer_dir + "/wq_a_w.bin", be.weight_bits(P["wq_a"]))
+        be.save(layer_dir + "/wq_a_y.bin", q_down)
+        be.save(layer_dir + "/q_norm_r.bin", q_down_rem)
+        be.save(layer_dir + "/q_norm_x.bin", q_down)
+        be.save(layer_dir + "/q_norm_weight.bin", be.weight_bits(P["q_norm"]))
+        be.save(layer_dir + "/q_norm_rms.bin", q_rms)
+        be.save(layer_dir + "/q_norm_y.bin", q_normed)
     q_nope, _ = be.linear(q_normed, P["wq_b1"], cq)
     q_pe, _ = be.linear(q_normed, P["wq_b2"], cq)
     q_nope = q_nope.reshape(1, S, H, cfg["nope"])
+    if layer_dir:                             # model.py:813-819 (q_pe_y.bin really receives the q_norm weights there)
+        be.save(layer_dir + "/q_pe_x.bin", q_pe.reshape(1, S, H, cfg["rope"]))
+        be.save("freqs_cis.bin", freqs)
+        be.save(layer_dir + "/q_pe_y.bin", be.weight_bits(P["q_norm"]))
     q_pe = q_pe.reshape(1, S, H, cfg["rope"] // 2, 2)
     q_pe = be.rope(q_pe, freqs).reshape(1, S, H, cfg["rope"])
-    kv, _ = be.linear(x, P["wkv_a1"], ckv)
+    kv, kv_rem = be.linear(x, P["wkv_a1"], ckv)
+    if layer_dir:                             # model.py:830-833
+        be.save(layer_dir + "/wkv_a1_x.bin", x)
+        be.save(layer_dir + "/wkv_a1_w.bin", be.weight_bits(P["wkv_a1"]))
+        be.save(layer_dir + "/wkv_a1_y.bin", kv)
+        be.save(layer_dir + "/wkv_a1_r.bin", kv_rem)
     k_pe, _ = be.linear(x, P["wkv_a2"], ckv)
     k_pe = be.rope(k_pe.reshape(1, S, 1, cfg["rope"] // 2, 2), freqs).reshape(1, S, cfg["rope"])
     q_abs = be.einsum("einsum_bshd_hdc_bshc", q_nope, P["wkv_b_1"], cfg["wkv_b_1_scale"])
     kv_normed = be.rmsnorm(kv[0], P["kv_norm"], cfg["kv_lora"])[None]
-    _, _, o = attention_scores_softmax_pv(be, q_abs, q_pe, kv_normed, k_pe)
+    _, _, o = attention_scores_softmax_pv(be, q_abs, q_pe, kv_normed, k_pe, layer_dir=layer_dir)
     o = be.einsum("einsum_bshc_hdc_bshd", o, P["wkv_b_2"], cfg["wkv_b_2_scale"])
     y, _ = be.linear(o.reshape(1, S, H * cfg["v"]), P["wo"], cfg["wo_scale"])
     return y
 
 
-def gate_scores(be, x, P, cfg):
+def gate_scores(be, x, P, cfg, layer_dir=None):
     """the kernel part of Gate.forward: linear at the gate's scale, then sigmoid_q23 (model.py:1116-1135)"""
-    s, _ = be.linear(x, P["gate"], cfg["gate_scale"])
-    return be.sigmoid(s)[0]
+    s, s_rem = be.linear(x, P["gate"], cfg["gate_scale"])
+    c = be.sigmoid(s)
+    if layer_dir:                             # model.py:1132-1138, 1151-1152
+        be.save(layer_dir + "/sigmoid_gate_x.bin", s)
+        be.save(layer_dir + "/sigmoid_gate_r.bin", s_rem)
+        be.save(layer_dir + "/sigmoid_gate_y.bin", c)
+        be.save(layer_dir + "/gate_original_scores.bin", c[0])
+        be.save(layer_dir + "/gate_bias.bin", P["gate_bias_host"].astype(np.int32))
+    return c[0]
 
 
 def route(scores_host, bias, cfg):
@@ -317,14 +439,25 @@ def route(scores_host, bias, cfg):
     return w, idx
 
 
-def moe(be, x, P, cfg):
+def moe(be, x, P, cfg, layer_dir=None):
     """MoE.forward (inference/model.py:1325-1383): shared expert + top-k routed experts, weights Q23"""
     T = x.shape[1]
-    sc = gate_scores(be, x, P, cfg)
-    w_host, idx_host = be.route(sc, P["gate_bias_host"], cfg) if hasattr(be, "route") else route(be.to_host(sc), P["gate_bias_host"], cfg)
+    shared = layer_dir + "/mlp_silu" if layer_dir else None
+    z = expert_ffn(be, x, P["sw1"], P["sw2"], P["sw3"], cfg["c13"], cfg["c2"], dump=shared)      # model.py:1346
+    sc = gate_scores(be, x, P, cfg, layer_dir)
+    if hasattr(be, "route"):
+        w_host, idx_host = be.route(sc, P["gate_bias_host"], cfg)
+        raw = be.last_raw_weights
+    else:
+        sc_host = be.to_host(sc)
+        w_host, idx_host = route(sc_host, P["gate_bias_host"], cfg)
+        raw = np.take_along_axis(sc_host, idx_host, axis=1)
+    if layer_dir:                             # model.py:1196-1197: the winners' unbiased scores, before they are normalised
+        be.save(layer_dir + "/gate_indices.bin", idx_host.astype(np.int64) if not hasattr(be, "route") else be.last_route[1])
+        be.save(layer_dir + "/gate_weights.bin", raw)
     if hasattr(be, "routed_experts"):
+        be.layer_dir = layer_dir
         y = be.routed_experts(x, P, cfg)
-        z = expert_ffn(be, x, P["sw1"], P["sw2"], P["sw3"], cfg["c13"], cfg["c2"])
         return y[None] + z, idx_host
     y = be.zeros_like(x[0])
     for e in range(cfg["experts"]):
@@ -332,17 +465,26 @@ def moe(be, x, P, cfg):
         if tok.size == 0:
             continue
         xe = x[0][be.from_host(tok)][None]
-        ye = expert_ffn(be, xe, P["w1"][e], P["w2"][e], P["w3"][e], cfg["c13"], cfg["c2"])[0]
+        ye = expert_ffn(be, xe, P["w1"][e], P["w2"][e], P["w3"][e], cfg["c13"], cfg["c2"],
+                        dump=layer_dir + "/expert_%d_silu" % e if layer_dir else None)[0]
         we = be.from_host(w_host[tok, slot].astype(np.int64))[:, None]
         y = be.index_add_rows(y, be.from_host(tok), (ye * we) // (1 << 23))      # model.py:1379
-    z = expert_ffn(be, x, P["sw1"], P["sw2"], P["sw3"], cfg["c13"], cfg["c2"])
     return y[None] + z, idx_host
 
 
-def decoder_layer(be, x, P, freqs, cfg):
-    """Block.forward for a MoE layer (inference/model.py:1430-1475): x Q31 residual stream [1,S,dim]"""
-    a = be.rmsnorm(x[0], P["attn_norm"], cfg["dim"])[None]
-    x, f = be.residual_rmsnorm(x[0], mla(be, a, P, freqs, cfg)[0], 12, P["ffn_norm"], cfg["dim"])   # model.py:1465-1468
+def decoder_layer(be, x, P, freqs, cfg, layer_dir=None):
+    """Block.forward for a MoE layer (inference/model.py:1430-1475): x Q31 residual stream [1,S,dim].  With `layer_dir`
+    (e.g. "pos_0/layer_3") and a back end whose `out` names a directory, the witness files the reference writes for
+    the layer are written under it, with the reference's names and bytes."""
+    a, a_rms = be.rmsnorm_with_statistic(x[0], P["attn_norm"], cfg["dim"])
+    a = a[None]
+    if layer_dir:                             # model.py:1455-1458
+        be.save(layer_dir + "/attn_norm_x.bin", x)
+        be.save(layer_dir + "/attn_norm_weight.bin", be.weight_bits(P["attn_norm"]))
+        be.save(layer_dir + "/attn_norm_y.bin", a)
+        be.save(layer_dir + "/attn_norm_rms.bin", a_rms)
+    x, f = be.residual_rmsnorm(x[0], mla(be, a, P, freqs, cfg, layer_dir)[0], 12, P["ffn_norm"], cfg["dim"])   # model.py:1465-1468
     x, f = x[None], f[None]
-    y, idx = moe(be, f, P, cfg)
+    y, idx = moe(be, f, P, cfg, layer_dir)
+    be.flush()
     return x + y * (1 << 8), idx                                 # model.py:1472

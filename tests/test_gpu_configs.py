@@ -115,6 +115,85 @@ def test_config5_decoder_layer_reduced(backends):
     kernel.lib.zk_gemm_set_path(0)
 
 
+def test_config5_witness_files_of_the_fused_layer(oracle, tmp_path):
+    """The product exists to write witnesses, and the proving side reads a fixed set of files per layer.  Config 5
+    reduced runs three times with the dump on: on the CPU restatement, on the GPU op by op with the reference's way of
+    saving (a synchronous copy and a file per tensor, inference/model.py:94-102), and on the GPU through the fused
+    entry points with the library's dump writer (device tensors handed over as they are, the statistic of the norms
+    left on the device, the per-expert files cut from the sorted intermediates).  The three directory trees must hold
+    the same files with the same bytes, and exactly the set the reference writes for a MoE layer
+    (inference/model.py:776-833, 913-918, 1037-1042, 1132-1152, 1196-1197, 1269-1274, 1455-1458)."""
+    import os
+    import kernel
+    kernel.lib.zk_gemm_set_path(0)
+    oracle.set_threads(oracle.max_threads())
+    cfg = dict(dim=512, q_lora=192, kv_lora=128, heads=8, nope=32, rope=16, v=32, experts=16, topk=4, groups=4,
+               topk_groups=2, inter=256, wkv_b_1_scale=31, wkv_b_2_scale=29, wo_scale=30, gate_scale=31, c13=30, c2=30)
+    g = torch.Generator(device="cpu").manual_seed(5100)
+    S = 24
+    i32 = torch.int32
+    w = lambda *shape: _ri(g, -(1 << 27), 1 << 27, shape, i32)
+    P = {
+        "attn_norm": _ri(g, 1 << 18, 1 << 20, (cfg["dim"],), i32), "ffn_norm": _ri(g, 1 << 18, 1 << 20, (cfg["dim"],), i32),
+        "q_norm": _ri(g, 1 << 18, 1 << 20, (cfg["q_lora"],), i32), "kv_norm": _ri(g, 1 << 20, 1 << 22, (cfg["kv_lora"],), i32),
+        "wq_a": w(cfg["q_lora"], cfg["dim"]), "wq_b1": w(cfg["heads"] * cfg["nope"], cfg["q_lora"]),
+        "wq_b2": w(cfg["heads"] * cfg["rope"], cfg["q_lora"]), "wkv_a1": w(cfg["kv_lora"], cfg["dim"]),
+        "wkv_a2": w(cfg["rope"], cfg["dim"]), "wkv_b_1": w(cfg["heads"], cfg["nope"], cfg["kv_lora"]),
+        "wkv_b_2": w(cfg["heads"], cfg["v"], cfg["kv_lora"]), "wo": w(cfg["dim"], cfg["heads"] * cfg["v"]),
+        "gate": w(cfg["experts"], cfg["dim"]),
+        "w1": [w(cfg["inter"], cfg["dim"]) for _ in range(cfg["experts"])],
+        "w3": [w(cfg["inter"], cfg["dim"]) for _ in range(cfg["experts"])],
+        "w2": [w(cfg["dim"], cfg["inter"]) for _ in range(cfg["experts"])],
+        "sw1": w(cfg["inter"], cfg["dim"]), "sw3": w(cfg["inter"], cfg["dim"]), "sw2": w(cfg["dim"], cfg["inter"]),
+    }
+    bias = _ri(g, -(1 << 18), 1 << 18, (cfg["experts"],)).numpy()
+    ang = torch.rand((1, S, 1, cfg["rope"] // 2), generator=g, dtype=torch.float64) * 6.283185307179586
+    freqs = torch.stack([torch.round(torch.cos(ang) * 2 ** 42), torch.round(torch.sin(ang) * 2 ** 42)], -1).to(torch.int64)
+    x = _ri(g, -(1 << 31), 1 << 31, (1, S, cfg["dim"]))
+
+    def place(fn):
+        out = {k: [fn(t) for t in v] if isinstance(v, list) else fn(v) for k, v in P.items()}
+        out["gate_bias_host"] = bias
+        return out
+
+    trees, outs = {}, {}
+    for name, be, fn in (("cpu", H.CpuBackend(oracle), lambda t: t.numpy()), ("kernels", H.GpuBackend(kernel), lambda t: t.cuda()),
+                         ("fused", H.FusedGpuBackend(kernel), lambda t: t.cuda())):
+        # the statistic buffer of the norms is returned whole, rows past the sequence included: same history for all
+        kernel.rms.zero_()
+        if kernel.rms_gpu is not None:
+            kernel.rms_gpu.zero_()
+        be.out = str(tmp_path / name)
+        y, idx = H.decoder_layer(be, fn(x), place(fn), fn(freqs), cfg, layer_dir="pos_0/layer_3")
+        outs[name] = (be.to_host(y), idx)
+        files = {}
+        for dirpath, _d, filenames in os.walk(be.out):
+            for f in filenames:
+                full = os.path.join(dirpath, f)
+                files[os.path.relpath(full, be.out)] = open(full, "rb").read()
+        trees[name] = files
+    oracle.set_threads(1)
+    hit = sorted(set(int(e) for e in outs["cpu"][1].reshape(-1)))
+    want = {"freqs_cis.bin"} | {"pos_0/layer_3/" + n + ".bin" for n in (
+        "attn_norm_x attn_norm_weight attn_norm_y attn_norm_rms wq_a_x wq_a_w wq_a_y q_norm_r q_norm_x q_norm_weight "
+        "q_norm_rms q_norm_y q_pe_x q_pe_y wkv_a1_x wkv_a1_w wkv_a1_y wkv_a1_r scores_softmax_x scores_softmax_y mlp_silu_x "
+        "mlp_silu_y sigmoid_gate_x sigmoid_gate_r sigmoid_gate_y gate_original_scores gate_bias gate_indices gate_weights").split()}
+    want |= {"pos_0/layer_3/expert_%d_silu_%s.bin" % (e, xy) for e in hit for xy in "xy"}
+    assert len(hit) > cfg["topk"] and len(hit) < cfg["experts"] + 1
+    for name, files in trees.items():
+        assert set(files) == want, (name, sorted(set(files) ^ want))
+    for f in sorted(want):
+        assert trees["kernels"][f] == trees["cpu"][f], "op-by-op GPU run differs from the CPU restatement in " + f
+        assert trees["fused"][f] == trees["kernels"][f], "fused GPU run differs from the op-by-op run in " + f
+    # sizes the proving side relies on: the statistic is the 500-row buffer, int32 weights are raw 4-byte words
+    t = trees["fused"]
+    assert len(t["pos_0/layer_3/attn_norm_rms.bin"]) == 500 * 8 and len(t["pos_0/layer_3/q_norm_rms.bin"]) == 500 * 8
+    assert len(t["pos_0/layer_3/wq_a_w.bin"]) == cfg["q_lora"] * cfg["dim"] * 4
+    assert len(t["pos_0/layer_3/gate_indices.bin"]) == S * cfg["topk"] * 8
+    assert sum(len(t["pos_0/layer_3/expert_%d_silu_x.bin" % e]) for e in hit) == S * cfg["topk"] * cfg["inter"] * 8
+    assert np.array_equal(outs["fused"][0], outs["cpu"][0]) and np.array_equal(outs["kernels"][0], outs["cpu"][0])
+
+
 def test_config5_decoder_layer_full_size(backends):
     """Config 5 at its real shape: one DeepSeek-V3 MoE decoder layer on 256 tokens, dim 7168, q_lora 1536, kv_lora
     512, 128 heads (nope 128 / rope 64 / v 128), 256 routed experts of width 2048 (top-8 in 4 of 8 groups) plus

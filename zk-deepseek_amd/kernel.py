@@ -526,10 +526,14 @@ def moe_combine(ye, weights, disp, T, shift=23):
     return y
 
 
-def moe_experts(x, weights, indices, w1_table, w3_table, w2_table, b32, inter, c13, c2):
+def moe_experts(x, weights, indices, w1_table, w3_table, w2_table, b32, inter, c13, c2, dump_dir=None):
     """The routed-expert part of MoE.forward (inference/model.py:1355-1381) without the Python loop: x [T,dim] Q23
     activations, (weights, indices) from the gate, pointer tables of the experts' w1/w3 [inter,dim] and w2 [dim,inter]
-    -> y [T,dim] = sum over each token's experts of (w2 . ((silu(w1 . x) * (w3 . x)) >> 23) * weight) >> 23."""
+    -> y [T,dim] = sum over each token's experts of (w2 . ((silu(w1 . x) * (w3 . x)) >> 23) * weight) >> 23.
+    dump_dir: the layer's witness directory.  The reference's Expert_int writes `expert_{i}_silu_x.bin` (w1 . x of the
+    expert's tokens, in token order) and `expert_{i}_silu_y.bin` (its SiLU) for every expert that has tokens
+    (inference/model.py:1269-1274); here they are the experts' segments of the sorted intermediates, handed to the dump
+    writer without a copy.  The segment table is read back for that (one wait, in dump mode only)."""
     T, dim = x.shape
     E = w1_table.numel()
     disp = moe_dispatch(indices.contiguous(), E)
@@ -537,7 +541,14 @@ def moe_experts(x, weights, indices, w1_table, w3_table, w2_table, b32, inter, c
     g = int64_grouped_bmm(xs, w1_table, b32, inter, c13, disp)
     u = int64_grouped_bmm(xs, w3_table, b32, inter, c13, disp)
     h = torch.empty_like(g)
-    silu_mul_q23(g.unsqueeze(0), u.unsqueeze(0), h.unsqueeze(0))
+    s = torch.empty_like(g) if dump_dir is not None else None
+    silu_mul_q23(g.unsqueeze(0), u.unsqueeze(0), h.unsqueeze(0), S=None if s is None else s.unsqueeze(0))
+    if dump_dir is not None:
+        seg = disp["seg"].cpu().tolist()
+        for i in range(E):
+            if seg[i + 1] > seg[i]:
+                saveTensor(os.path.join(dump_dir, "expert_%d_silu_x.bin" % i), g[seg[i]:seg[i + 1]])
+                saveTensor(os.path.join(dump_dir, "expert_%d_silu_y.bin" % i), s[seg[i]:seg[i + 1]])
     ye = int64_grouped_bmm(h, w2_table, b32, dim, c2, disp)
     return moe_combine(ye, weights.contiguous(), disp, T)
 
