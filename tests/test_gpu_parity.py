@@ -97,6 +97,25 @@ def test_gemm_many_digit_operands_at_every_shift(K, oracle, bits_a, bits_w, w32,
     K.lib.zk_gemm_set_path(0)
 
 
+@pytest.mark.parametrize("Kd", [14560, 14600, 16384, 18432])
+def test_gemm_long_k_with_nine_digit_operands(K, oracle, Kd):
+    """the int32 accumulators of the MFMA path hold min(NA, NB) * K * 2^14: with nine digits that ends at K = 14563.
+    Beyond it every tile is split along K (partial sums, then the finishing kernel) instead of falling back to the
+    vector ALU; operands whose digits all sit at their extremes, on both sides of the bound and at the model's 16384 /
+    18432"""
+    rng = np.random.default_rng(Kd)
+    A = rand_i64(rng, (1, 70, Kd), 63)
+    W = rand_i64(rng, (150, Kd), 63)
+    A[0, 0, :] = -0x7F7F7F7F7F7F7F80 - 1            # every digit -128 (and the ninth 0): the largest products
+    A[0, 1, :] = 0x7F7F7F7F7F7F7F7F
+    W[0, :] = -0x7F7F7F7F7F7F7F80 - 1
+    W[1, :] = 0x7F7F7F7F7F7F7F7F
+    for c in (0, 29, 63):
+        _gemm_case(K, oracle, 2, A, W, 1, 1, c)
+        assert K.gemm_last_plan() == (2, 9, 9), "the long K must stay on the MFMA path"
+    K.lib.zk_gemm_set_path(0)
+
+
 @pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 1, 7, 1), (3, 5, 17, 9), (1, 64, 64, 64), (1, 65, 129, 63),
                                    (1, 128, 32, 256), (2, 33, 1000, 31), (1, 257, 96, 130)])

@@ -550,7 +550,8 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         // int32 accumulators: at most min(NA,NB) digit pairs per diagonal, each product at most 2^14 in magnitude
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
         const int ksteps = ((d.K + 32 * inst->kk - 1) / (32 * inst->kk)) * inst->kk;     // 32-k steps, padded
-        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return kDeclined;
+        // (a K beyond that bound is cut into slices that respect it: every tile is then split, see below)
+        const bool k_over = pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL;
         const int BM = inst->bm, BN = inst->bn;
         p.tiles_m = (d.M + BM - 1) / BM;
         p.tiles_n = (d.N + BN - 1) / BN;
@@ -605,6 +606,19 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                 if (split > steps / 8) split = steps / 8;
             }
         }
+        if (k_over) {
+            // every tile in slices short enough for the int32 accumulators; without room for the partial sums (or with
+            // the split switched off) the vector-ALU path takes the product
+            int min_split = 2;
+            while (pairs * ((steps + min_split - 1) / min_split) * 32 * inst->kk * 16384 > 0x7FFFFFFFL) min_split++;
+            if (g_switches.no_tail_split || min_split > steps) return kDeclined;
+            if (tail != (int)total || split < min_split) {
+                tail = (int)total;
+                split = min_split;
+                p.finish_rq = 4;
+            }
+            if ((size_t)tail * split * BM * BN * 16 > ((size_t)2 << 30)) return kDeclined;
+        }
         if (split >= 2) {
             // |sum| < K * 2^(8(NA+NB)-2): below 2^62 the low word alone carries a partial sum
             int kbits = 0;
@@ -620,6 +634,7 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                 p.partials = g_cache.partials;
                 p.part64 = part64 ? 1 : 0;
             } else if (got == kFailed) return kFailed;
+            else if (k_over) return kDeclined;
         }
         const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
         if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;
