@@ -473,27 +473,46 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
         for (int r = 0; r < 4; r++) slot[(ct * 4 + r) * 64 + lane] = sums[ct][r];
 }
 
-// Adds the slots of every output tile, applies rounding term and shift, stores C and R: one thread per output.
+// Adds the slots of every output tile, applies rounding term and shift, stores C and R.  Four threads share an output
+// (each adds every fourth slice with all its loads under way at once, then the four meet through shuffles): the launch
+// is a chain of one load latency, not of one per slice.
 template <bool B32>
 __global__ __launch_bounds__(256) void gemm_rows16_finish_kernel(Rows16Params p)
 {
     constexpr int CT = R16Shape<B32>::kColTiles, PER = CT * 4 * 64;         // sums per slot
-    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long idx = ((long)blockIdx.x * 256 + threadIdx.x) >> 2;
+    const int part = threadIdx.x & 3;
     const long tile_id = idx / PER;
     const int o = (int)(idx - tile_id * PER), lane = o & 63, cr = o >> 6, ct = cr >> 2, r = cr & 3;
     const long tiles = (long)p.G * p.row_tiles * p.col_groups;
-    if (tile_id >= tiles) return;
+    if (tile_id >= tiles) return;                                          // (whole groups of four leave together)
     const int cg = (int)(tile_id % p.col_groups);
     const long t2 = tile_id / p.col_groups;
     const int rt = (int)(t2 % p.row_tiles), g = (int)(t2 / p.row_tiles);
     const int m = rt * 16 + 4 * (lane >> 4) + r, n = cg * R16Shape<B32>::kCols + 16 * ct + (lane & 15);
-    if (m >= p.M || n >= p.N) return;
     const int groups = p.nslices;
     const u128 *slot = reinterpret_cast<const u128 *>(p.acc) + tile_id * groups * PER + o;
-    u128 s = (u128)(i128)p.init;
-#pragma unroll 8
-    for (int gi = 0; gi < groups; gi++) s += slot[(long)gi * PER];
-    const uint64_t lo = (uint64_t)s, hi = (uint64_t)(s >> 64);
+    u128 s = 0;
+    for (int g0 = part; g0 < groups; g0 += 32) {
+        u128 t[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = g0 + 4 * j < groups ? slot[(long)(g0 + 4 * j) * PER] : (u128)0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) s += t[j];
+    }
+    uint64_t lo = (uint64_t)s, hi = (uint64_t)(s >> 64);
+#pragma unroll
+    for (int off = 1; off < 4; off <<= 1) {
+        const uint64_t olo = (uint64_t)__shfl_xor((long long)lo, off, 64), ohi = (uint64_t)__shfl_xor((long long)hi, off, 64);
+        const uint64_t tlo = lo + olo;
+        hi += ohi + (tlo < lo ? 1 : 0);
+        lo = tlo;
+    }
+    if (part != 0 || m >= p.M || n >= p.N) return;
+    const uint64_t ilo = (uint64_t)p.init, ihi = (uint64_t)(p.init >> 63);
+    const uint64_t flo = lo + ilo;
+    hi += ihi + (flo < lo ? 1 : 0);
+    lo = flo;
     const long at = (long)g * p.sC + (long)m * p.ldc + n;
     p.C[at] = (int64_t)((lo >> p.shift) | ((hi << 1) << (63 - p.shift)));
     if (p.R) p.R[at] = (int64_t)(p.shift ? lo & ((1ull << p.shift) - 1) : 0);
@@ -632,7 +651,7 @@ int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_sl
     }
     const int rc = r16_run(d.b32 ? gemm_rows16_kernel<true, false> : gemm_rows16_kernel<false, false>, p, wg_tiles * p.nslices);
     if (rc != 0 || p.nslices == 1) return rc;
-    const long threads = tiles * (d.b32 ? R16Shape<true>::kColTiles : R16Shape<false>::kColTiles) * 4 * 64;
+    const long threads = tiles * (d.b32 ? R16Shape<true>::kColTiles : R16Shape<false>::kColTiles) * 4 * 64 * 4;      // four per output
     const dim3 grid((unsigned)((threads + 255) / 256));
     if (d.b32) gemm_rows16_finish_kernel<true><<<grid, dim3(256), 0, 0>>>(p);
     else gemm_rows16_finish_kernel<false><<<grid, dim3(256), 0, 0>>>(p);
