@@ -444,7 +444,18 @@ def run():
         for Tt in (256, 65536):
             gsc = randint(gr, 1, 1 << 23, (Tt, 256)).cuda()
             hbm("gate_route_%dx256" % Tt, lambda: K.gate_route(gsc, gbias, 8, 4, 8), Tt, bytes_per_elem=8.0 * 256 + 128.0, steps=20)
-            del gsc
+            # sigmoid and routing in one launch, from the gate's logits (the scores not written: the same bytes)
+            glog = randint(gr, -(1 << 25), 1 << 25, (Tt, 256)).cuda()
+            hbm("gate_sigmoid_route_%dx256" % Tt, lambda: K.gate_sigmoid_route(glog, gbias, 8, 4, 8, keep_scores=False), Tt,
+                bytes_per_elem=8.0 * 256 + 128.0, steps=20)
+            gsig = torch.empty_like(glog)
+
+            def two_launches():
+                K.sigmoid_q23(glog[None], gsig[None])
+                K.gate_route(gsig, gbias, 8, 4, 8)
+
+            extra["gate_sigmoid_route_%dx256" % Tt]["unfused_chain_ms"] = timed(K, two_launches, 20, 3)
+            del gsc, glog, gsig
 
         # config 5's routed experts: 256 tokens, top 8 of 256 experts of width 2048 on dim 7168, int64 weights resident
         # (90.2 GB): bound by the one pass over the weights.  Routing, dispatch, three grouped GEMM launches, combine.

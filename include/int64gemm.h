@@ -162,6 +162,14 @@ void silu_mul_q23(const int64_t *R, const int64_t *U, int64_t *S, int64_t *C, co
 void gate_route_q23(const int64_t *scores, const int32_t *bias, int64_t *weights, int64_t *indices,
                     int64_t *raw_weights, int T, int E, int n_groups, int topk_groups, int topk);
 
+/* The same routing straight from the gate's logits (no counterpart in the reference's library; it replaces sigmoid_q23
+ * plus the tensor ops of inference/model.py:1135-1208 by one launch): every logit goes through sigmoid_q23 (table `lut`,
+ * 256 entries as the silu/sigmoid kernels take it) first.  scores [T,E] (may be null) receives the sigmoid values, i.e.
+ * what gate_route_q23 takes as input and the reference dumps as sigmoid_gate_y.bin / gate_original_scores.bin. */
+void gate_sigmoid_route_q23(const int64_t *logits, const int64_t *lut, const int32_t *bias, int64_t *scores,
+                            int64_t *weights, int64_t *indices, int64_t *raw_weights, int T, int E, int n_groups,
+                            int topk_groups, int topk);
+
 /* Witness dump writer (replaces the reference's saveTensor, inference/model.py:94-102: a synchronous .cpu() copy and
  * file write per tensor, ~30 per layer).  zk_dump_device queues the raw bytes of `bytes` bytes of contiguous device
  * memory for `path`: the copy to pinned host memory is ordered on the null stream behind the kernels that produced

@@ -224,10 +224,23 @@ class FusedGpuBackend(GpuBackend):
     def flush(self):
         self.k.dump_flush()
 
-    def route(self, scores, bias_host, cfg):
+    def sigmoid_route(self, logits, bias_host, cfg):
+        """sigmoid and routing in one launch: returns the sigmoid scores, keeps the routing for route()"""
         bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
-        raw = self.t.empty((scores.shape[0], cfg["topk"]), dtype=self.t.int64, device="cuda")
-        w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"], raw_weights=raw)
+        raw = self.t.empty((logits.shape[1], cfg["topk"]), dtype=self.t.int64, device="cuda")
+        sc, w, idx = self.k.gate_sigmoid_route(logits[0].contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"],
+                                               raw_weights=raw)
+        self._routed = (w, idx, raw)
+        return sc[None]
+
+    def route(self, scores, bias_host, cfg):
+        if getattr(self, "_routed", None) is not None:
+            w, idx, raw = self._routed
+            self._routed = None
+        else:
+            bias = self.t.from_numpy(bias_host.astype(np.int32)).cuda()
+            raw = self.t.empty((scores.shape[0], cfg["topk"]), dtype=self.t.int64, device="cuda")
+            w, idx = self.k.gate_route(scores.contiguous(), bias, cfg["groups"], cfg["topk_groups"], cfg["topk"], raw_weights=raw)
         self.last_route = (w, idx)
         self.last_raw_weights = raw
         return w.cpu().numpy(), idx.cpu().numpy()
@@ -409,7 +422,7 @@ def mla(be, x, P, freqs, cfg, layer_dir=None):
 def gate_scores(be, x, P, cfg, layer_dir=None):
     """the kernel part of Gate.forward: linear at the gate's scale, then sigmoid_q23 (model.py:1116-1135)"""
     s, s_rem = be.linear(x, P["gate"], cfg["gate_scale"])
-    c = be.sigmoid(s)
+    c = be.sigmoid_route(s, P["gate_bias_host"], cfg) if hasattr(be, "sigmoid_route") else be.sigmoid(s)
     if layer_dir:                             # model.py:1132-1138, 1151-1152
         be.save(layer_dir + "/sigmoid_gate_x.bin", s)
         be.save(layer_dir + "/sigmoid_gate_r.bin", s_rem)

@@ -1041,12 +1041,19 @@ def test_silu_mul_q23_fusion(K, oracle, shape, keep):
         assert np.array_equal(host(S), se)
 
 
-@pytest.mark.parametrize("E,G,KG,K_", [(256, 8, 4, 8), (16, 4, 2, 4), (64, 1, 1, 6), (96, 3, 3, 5), (512, 8, 3, 8), (1024, 16, 5, 64), (7, 1, 1, 7)])
+# (the shapes with 2..16 groups of 8, 16 or 32 experts run on the lane-per-group kernel, the others on the wave-wide one;
+#  (64, 8, 2, 40) and (32, 2, 1, 20) ask for more winners than the kept groups hold, so masked experts win too)
+GATE_SHAPES = [(256, 8, 4, 8), (16, 4, 2, 4), (64, 1, 1, 6), (96, 3, 3, 5), (512, 8, 3, 8), (1024, 16, 5, 64), (7, 1, 1, 7),
+               (512, 16, 4, 6), (64, 4, 2, 9), (64, 8, 2, 40), (32, 2, 1, 20), (128, 16, 16, 64), (64, 2, 2, 3)]
+
+
+@pytest.mark.parametrize("E,G,KG,K_", GATE_SHAPES)
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gate_route(K, oracle, E, G, KG, K_, with_bias):
     """routing of Gate.forward on the device against the oracle, ties included (coarse scores tie often)"""
     rng = np.random.default_rng(E * 3 + G + with_bias)
-    for T, hi in ((1, 1 << 23), (77, 1 << 23), (300, 12)):
+    # (beyond 8192 tokens the lane-per-group kernel switches from four lanes per group to one)
+    for T, hi in ((1, 1 << 23), (77, 1 << 23), (300, 12), (1031, 1 << 23), (8200, 1 << 23), (8195, 9)):
         scores = rng.integers(1, hi, size=(T, E), dtype=np.int64)
         bias = rng.integers(-(hi >> 3) - 1, (hi >> 3) + 1, size=E, dtype=np.int64).astype(np.int32) if with_bias else None
         raw = torch.empty((T, K_), dtype=torch.int64, device="cuda")
@@ -1055,6 +1062,28 @@ def test_gate_route(K, oracle, E, G, KG, K_, with_bias):
         assert np.array_equal(host(idx), ie), "indices"
         assert np.array_equal(host(raw), re_), "gathered scores"
         assert np.array_equal(host(w), we), "weights"
+
+
+@pytest.mark.parametrize("E,G,KG,K_", GATE_SHAPES)
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_gate_sigmoid_route(K, oracle, E, G, KG, K_, with_bias):
+    """sigmoid and routing in one launch against the oracle's sigmoid_q23 followed by its routing: logits over the
+    sigmoid's whole domain (the ends saturate, so scores tie), with and without the scores written"""
+    rng = np.random.default_rng(E * 5 + G + with_bias)
+    for T, span in ((1, 1 << 26), (130, 1 << 24), (515, 1 << 31), (64, 40), (8197, 1 << 25)):
+        logits = rng.integers(-span, span, size=(T, E), dtype=np.int64)
+        bias = rng.integers(-(1 << 20), 1 << 20, size=E, dtype=np.int64).astype(np.int32) if with_bias else None
+        sig = oracle.sigmoid_q23(logits[None])[0]
+        we, ie, re_ = oracle.gate_route(sig, bias, G, KG, K_)
+        for keep in (True, False):
+            raw = torch.empty((T, K_), dtype=torch.int64, device="cuda")
+            sc, w, idx = K.gate_sigmoid_route(dev(logits), None if bias is None else dev(bias), G, KG, K_, raw, keep_scores=keep)
+            assert (sc is None) == (not keep)
+            if keep:
+                assert np.array_equal(host(sc), sig), "sigmoid scores"
+            assert np.array_equal(host(idx), ie), "indices"
+            assert np.array_equal(host(raw), re_), "gathered scores"
+            assert np.array_equal(host(w), we), "weights"
 
 
 def _routing(rng, T, E, Kr):

@@ -78,6 +78,7 @@ lib.zk_gemm_grouped_mfma_calls.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
 lib.gate_route_q23.argtypes = [_vp] * 5 + [_ci] * 5
+lib.gate_sigmoid_route_q23.argtypes = [_vp] * 7 + [_ci] * 5
 lib.moe_dispatch.argtypes = [_vp, _ci, _ci, _ci] + [_vp] * 6
 lib.moe_gather_rows.argtypes = [_vp, _vp, _vp, _ci, _ci]
 lib.int64_grouped_bmm_launcher.argtypes = [_vp, _vp, _ci, _vp, _vp, ctypes.c_longlong, _vp, _vp, _vp, _ci, _ci, _ci, _ci]
@@ -469,6 +470,24 @@ def gate_route(scores, bias, n_groups, topk_groups, topk, raw_weights=None):
                        0 if raw_weights is None else raw_weights.data_ptr(), T, E, n_groups, topk_groups, topk)
     _check("gate_route_q23")
     return weights, indices
+
+
+def gate_sigmoid_route(logits, bias, n_groups, topk_groups, topk, raw_weights=None, keep_scores=True):
+    """sigmoid_q23 and the routing of Gate.forward in one launch (inference/model.py:1135-1208): logits [T,E] int64 (the
+    gate's linear output, Q23) -> (scores [T,E] or None, weights [T,topk], indices [T,topk]).  `scores` is what the
+    reference keeps as original_scores and dumps as sigmoid_gate_y.bin; keep_scores=False skips writing it."""
+    assert logits.is_cuda and logits.dtype == torch.int64 and logits.is_contiguous() and logits.dim() == 2
+    assert bias is None or (bias.is_cuda and bias.dtype == torch.int32 and bias.is_contiguous() and bias.numel() == logits.shape[1])
+    assert EXP2_FRAC_LUT_Q23 is not None, "call silu_init_q23 first"
+    T, E = logits.shape
+    scores = torch.empty_like(logits) if keep_scores else None
+    weights = torch.empty((T, topk), dtype=torch.int64, device=logits.device)
+    indices = torch.empty((T, topk), dtype=torch.int64, device=logits.device)
+    lib.gate_sigmoid_route_q23(logits.data_ptr(), EXP2_FRAC_LUT_Q23.data_ptr(), 0 if bias is None else bias.data_ptr(),
+                               0 if scores is None else scores.data_ptr(), weights.data_ptr(), indices.data_ptr(),
+                               0 if raw_weights is None else raw_weights.data_ptr(), T, E, n_groups, topk_groups, topk)
+    _check("gate_sigmoid_route_q23")
+    return scores, weights, indices
 
 
 # ---- MoE dispatch on the device (replaces the Python loop over the experts of MoE.forward, model.py:1325-1383)
