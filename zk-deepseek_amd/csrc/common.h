@@ -29,6 +29,11 @@ void act_release_workspace();
 
 constexpr int kWave = 64;
 
+// A pointer that came out of memory itself (an expert's matrix from the table of a grouped launch) could point anywhere
+// as far as the compiler knows, and a load through it counts as an LDS access as well: every wait for LDS then waits
+// for the weights under way.  Loads of operands name their address space: (const ZK_GLOBAL_MEM T *)ptr.
+#define ZK_GLOBAL_MEM __attribute__((address_space(1)))
+
 // ---- wave-level helpers --------------------------------------------------------------------
 // 64-lane butterfly reductions.  Every lane ends up with the result.
 __device__ __forceinline__ int64_t wave_max_i64(int64_t v)

@@ -206,14 +206,15 @@ __device__ __forceinline__ int owned_k(int j, int e) { return RUN * OCTS * (e / 
 
 // Loads the 8 owned int64 elements of one row; `src` points at the row's first k of this step.
 template <int RUN, int OCTS>
-__device__ __forceinline__ void load_owned_i64(const int64_t *src, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
+__device__ __forceinline__ void load_owned_i64(const int64_t *src_generic, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
 {
+    const ZK_GLOBAL_MEM int64_t *src = (const ZK_GLOBAL_MEM int64_t *)src_generic;
     if (row_ok && owned_k<RUN, OCTS>(j, 7) < k_left && vec) {
 #pragma unroll
         for (int q = 0; q < 8 / RUN; q++) {
 #pragma unroll
             for (int h = 0; h < RUN / 2; h++) {
-                const v4i t = *reinterpret_cast<const v4i *>(src + owned_k<RUN, OCTS>(j, q * RUN + 2 * h));
+                const v4i t = *(const ZK_GLOBAL_MEM v4i *)(src + owned_k<RUN, OCTS>(j, q * RUN + 2 * h));
                 x[q * RUN + 2 * h] = (int64_t)(((uint64_t)(uint32_t)t[1] << 32) | (uint32_t)t[0]);
                 x[q * RUN + 2 * h + 1] = (int64_t)(((uint64_t)(uint32_t)t[3] << 32) | (uint32_t)t[2]);
             }
@@ -228,12 +229,13 @@ __device__ __forceinline__ void load_owned_i64(const int64_t *src, int j, bool r
 }
 
 template <int RUN, int OCTS>
-__device__ __forceinline__ void load_owned_i32(const int32_t *src, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
+__device__ __forceinline__ void load_owned_i32(const int32_t *src_generic, int j, bool row_ok, int k_left, bool vec, int64_t (&x)[8])
 {
+    const ZK_GLOBAL_MEM int32_t *src = (const ZK_GLOBAL_MEM int32_t *)src_generic;
     if (RUN == 4 && row_ok && owned_k<RUN, OCTS>(j, 7) < k_left && vec) {
 #pragma unroll
         for (int q = 0; q < 2; q++) {
-            const v4i t = *reinterpret_cast<const v4i *>(src + owned_k<RUN, OCTS>(j, q * 4));
+            const v4i t = *(const ZK_GLOBAL_MEM v4i *)(src + owned_k<RUN, OCTS>(j, q * 4));
 #pragma unroll
             for (int z = 0; z < 4; z++) x[q * 4 + z] = (int64_t)t[z];
         }
@@ -502,7 +504,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     v4i pa[A_CIT], pb[B_CIT];
 
     const bool a_vec = (((uintptr_t)p.A | (uintptr_t)(p.lda * 8) | (uintptr_t)(p.sA * 8)) & 15) == 0;
-    const bool b_vec = BPL || !BKM && (((uintptr_t)b_base | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0;
+    const bool b_vec = BPL || (!BKM && (((uintptr_t)b_base | (uintptr_t)(p.ldbn * (B32 ? 4 : 8)) | (uintptr_t)(p.sB * (B32 ? 4 : 8))) & 15) == 0);
 
     // per-thread source pointers (advanced by BK per step) and LDS destinations
     const int64_t *a_src[A_IT];
@@ -591,7 +593,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         if (BPL) {
 #pragma unroll
             for (int it = 0; it < B_CIT; it++)
-                pb[it] = *reinterpret_cast<const v4i *>(b_pl[it] + (long)ks * (KK * NB * 1024));
+                pb[it] = *(const ZK_GLOBAL_MEM v4i *)(b_pl[it] + (long)ks * (KK * NB * 1024));
         }
 #pragma unroll
         for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
@@ -602,8 +604,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
                     const long off = (long)k * p.ldbk;
                     int64_t v = 0;
                     if (FAST || k < p.K)
-                        v = B32 ? (int64_t)reinterpret_cast<const int32_t *>(b_src[it])[off]
-                                : reinterpret_cast<const int64_t *>(b_src[it])[off];
+                        v = B32 ? (int64_t)((const ZK_GLOBAL_MEM int32_t *)b_src[it])[off] : ((const ZK_GLOBAL_MEM int64_t *)b_src[it])[off];
                     sb[it][e] = v;
                 }
             } else if (B32) {

@@ -13,6 +13,9 @@
 
 namespace zk {
 
+typedef int v4i_g __attribute__((ext_vector_type(4)));
+typedef long long v2l_g __attribute__((ext_vector_type(2)));
+
 constexpr int kVT = 64;        // tile edge (rows of A and of B per workgroup)
 constexpr int kVK = 16;        // k-steps per LDS stage
 constexpr int kVP = 68;        // padded row length of the [k][row] LDS tiles (int64 units)
@@ -264,11 +267,11 @@ __global__ __launch_bounds__(256) void gemv_kernel(ValuParams p)
                     for (int e = 0; e < EPL; e++) b[u][c][e] = 0;
                     if (in) {
                         if (B32) {
-                            const int4 t = *reinterpret_cast<const int4 *>(reinterpret_cast<const int32_t *>(Bbase) + brow[c] + 4 * q);
-                            b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y; b[u][c][2 % EPL] = (BT)t.z; b[u][c][3 % EPL] = (BT)t.w;
+                            const v4i_g t = *(const ZK_GLOBAL_MEM v4i_g *)(reinterpret_cast<const int32_t *>(Bbase) + brow[c] + 4 * q);
+                            b[u][c][0] = (BT)t[0]; b[u][c][1] = (BT)t[1]; b[u][c][2 % EPL] = (BT)t[2]; b[u][c][3 % EPL] = (BT)t[3];
                         } else {
-                            const longlong2 t = *reinterpret_cast<const longlong2 *>(reinterpret_cast<const int64_t *>(Bbase) + brow[c] + 2 * q);
-                            b[u][c][0] = (BT)t.x; b[u][c][1] = (BT)t.y;
+                            const v2l_g t = *(const ZK_GLOBAL_MEM v2l_g *)(reinterpret_cast<const int64_t *>(Bbase) + brow[c] + 2 * q);
+                            b[u][c][0] = (BT)t[0]; b[u][c][1] = (BT)t[1];
                         }
                     }
                 }
@@ -411,7 +414,7 @@ __global__ __launch_bounds__(64 * kStagedWaves) void gemv32_staged_kernel(ValuPa
 #pragma unroll
         for (int c = 0; c < CPW; c++) {
             const long n = n_first + c < p.N ? n_first + c : p.N - 1;      // columns past N read the last row; dropped below
-            const v4i_s *brow = reinterpret_cast<const v4i_s *>(Bbase + n * p.ldbn + k0);
+            const ZK_GLOBAL_MEM v4i_s *brow = (const ZK_GLOBAL_MEM v4i_s *)(Bbase + n * p.ldbn + k0);
             for (int q0 = 0; q0 < units; q0 += 64 * UN) {
                 v4i_s b[UN];
 #pragma unroll

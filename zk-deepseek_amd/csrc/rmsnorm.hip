@@ -72,11 +72,34 @@ __device__ __forceinline__ U192 wave_sum_u192(U192 a)
     return a;
 }
 
-// floor(x / d), d > 0.  32-bit divisors (every model shape) use schoolbook division on 32-bit digits.
+// floor(x / d), d > 0.  32-bit divisors use schoolbook division on 32-bit digits; below 2^20 (every model shape:
+// the row length) a digit step is a double-precision estimate and one correction.  This runs on one lane while the
+// rest of the row's workgroup waits, so its length is the latency of a short launch.
 __device__ U192 u192_div(U192 x, uint64_t d)
 {
     U192 q;
-    if (d <= 0xFFFFFFFFull) {
+    if (d < (1ull << 20)) {
+        const uint32_t dig[6] = { (uint32_t)x.w0, (uint32_t)(x.w0 >> 32), (uint32_t)x.w1,
+                                  (uint32_t)(x.w1 >> 32), (uint32_t)x.w2, (uint32_t)(x.w2 >> 32) };
+        uint32_t qd[6];
+        const double inv = 1.0 / (double)d;
+        uint64_t rem = 0;
+#pragma unroll
+        for (int i = 5; i >= 0; i--) {
+            // cur < 2^52 is exact as a double and cur / d < 2^32: the estimate is off by less than 2^-20, its floor by
+            // at most one either way
+            const uint64_t cur = (rem << 32) | dig[i];
+            uint64_t qi = (uint64_t)((double)cur * inv);
+            int64_t r = (int64_t)(cur - qi * d);
+            if (r < 0) { qi--; r += (int64_t)d; }
+            else if (r >= (int64_t)d) { qi++; r -= (int64_t)d; }
+            qd[i] = (uint32_t)qi;
+            rem = (uint64_t)r;
+        }
+        q.w0 = qd[0] | ((uint64_t)qd[1] << 32);
+        q.w1 = qd[2] | ((uint64_t)qd[3] << 32);
+        q.w2 = qd[4] | ((uint64_t)qd[5] << 32);
+    } else if (d <= 0xFFFFFFFFull) {
         uint32_t dig[6] = { (uint32_t)x.w0, (uint32_t)(x.w0 >> 32), (uint32_t)x.w1,
                             (uint32_t)(x.w1 >> 32), (uint32_t)x.w2, (uint32_t)(x.w2 >> 32) };
         uint32_t qd[6];
