@@ -504,6 +504,25 @@ def run():
                 hbm(nm, lambda: K.moe_experts(xt, wt, it, tabs[0], tabs[1], tabs[2], True, 2048, 30, 33), 1, bytes_per_elem=wbytes, steps=3)
                 extra[nm]["weight_bytes"] = wbytes
                 extra[nm]["experts_hit"] = hit
+                if Tt == 256:
+                    # The same with activation buffers the library has not seen: the legs above hand it the same
+                    # addresses call after call (torch's allocator returns them), so its remembered digit counts hit.
+                    # Here every call's intermediates land on new memory (a growing pile of blocks keeps the old
+                    # addresses taken): what a layer pays whose buffers move.  Wall clock, since such a call waits.
+                    pile = []
+
+                    def fresh_call():
+                        pile.append(torch.empty((Tt * 8 * 7168 + 4096 * len(pile),), dtype=torch.int64, device="cuda"))
+                        return K.moe_experts(xt, wt, it, tabs[0], tabs[1], tabs[2], True, 2048, 30, 33)
+
+                    fresh_call()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(3):
+                        fresh_call()
+                    torch.cuda.synchronize()
+                    extra[nm]["ms_with_activation_buffers_at_new_addresses"] = (time.perf_counter() - t0) * 1e3 / 3
+                    del pile
             # 256 tokens again with the int32 weights prepared as digit planes (four bytes per weight, as before, but
             # nothing of B is split in the kernel)
             torch.cuda.synchronize()

@@ -111,8 +111,8 @@ void zk_clear_error(void);
 size_t zk_workspace_bytes(void);
 size_t zk_prepared_weights_bytes(void);
 void zk_release_workspace(void);
-/* Reads the diagnosis switches ZK_GEMM_SYNC, ZK_NO_TAIL_SPLIT and ZK_B_ROWS_MIN_MACS from the environment again (they
- * are read once when the library is loaded, not per call). */
+/* Reads the diagnosis switches ZK_GEMM_SYNC, ZK_NO_TAIL_SPLIT, ZK_B_ROWS_MIN_MACS and ZK_ROWS16_MAX_WEIGHTS from the
+ * environment again (they are read once when the library is loaded, not per call). */
 void zk_reload_env(void);
 
 /* RMS statistic on the device: rms[m] = isqrt((eps + sum_n A[m,n]^2) / dim), exact (192-bit sum).

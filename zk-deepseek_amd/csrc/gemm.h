@@ -48,6 +48,7 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b);
 int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc = nullptr, size_t max_slots = 0);
 size_t gemm_rows16_workspace_bytes();
 void gemm_rows16_release_workspace();
+void gemm_rows16_reload_switches();
 
 // Calls of the MFMA path that returned before their verdict was known and turned out to need the guarded
 // vector-ALU recomputation (known once their range has reached the host).

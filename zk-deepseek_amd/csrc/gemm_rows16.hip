@@ -26,6 +26,8 @@
 // the slots, applies rounding term and shift and stores.
 #include "gemm_mfma_kernels.h"
 
+#include <cstdlib>
+
 namespace zk {
 
 struct Rows16Params {
@@ -627,11 +629,25 @@ static int r16_run(Rows16Kernel fn, const Rows16Params &p, long blocks)
     return 0;
 }
 
+// Matrices with more weights than this go to the 32-row kernels instead (the library's own calls only): a stream that
+// long is bound by the bytes in flight per compute unit, which LDS caps at 96 KB here.  Measured with 16 rows, both
+// weight types: 14.7 M weights ([2048,7168]) 0.79-0.97 of the 32-row kernels' time, 29 M 1.09-1.12, 132 M 1.37-1.48.
+// ZK_ROWS16_MAX_WEIGHTS overrides.
+constexpr long kR16MaxWeights = 20L << 20;
+static long r16_read_limit()
+{
+    const char *e = getenv("ZK_ROWS16_MAX_WEIGHTS");
+    return e ? atol(e) : kR16MaxWeights;
+}
+static long g_r16_max_weights = r16_read_limit();
+void gemm_rows16_reload_switches() { g_r16_max_weights = r16_read_limit(); }
+
 // acc: scratch for split K (`max_slots` slots of 8 KB); null: the library's own, grown on demand
 int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_slots)
 {
     Rows16Params p;
     if (!r16_fill(d, p)) return 1;
+    if (!acc && (long)d.N * d.K > g_r16_max_weights) return 1;
     const long tiles = (long)d.G * p.row_tiles * p.col_groups;
     const long wg_tiles = (long)d.G * p.row_tiles * ((p.col_groups + kR16Waves - 1) / kR16Waves);
     if (tiles > (1L << 24)) return 1;

@@ -106,7 +106,11 @@ void zk_release_workspace(void)
     zk::act_release_workspace();
 }
 
-void zk_reload_env(void) { zk::gemm_mfma_reload_switches(); }
+void zk_reload_env(void)
+{
+    zk::gemm_mfma_reload_switches();
+    zk::gemm_rows16_reload_switches();
+}
 
 void zk_timer_start(void)
 {
