@@ -718,7 +718,10 @@ def run():
         wbytes = 8.0 * (576 * 7168 + 16 * 7168 + 2 * 16 * 576)
         gbs = wbytes / (e["ms"] * 1e-3) / 1e9
         others["gemm_config1_16x7168x576"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                                              "traffic": None, "note": "algorithmic bytes 8*(N*K + M*K + 2*M*N) = %.0f per call: the weights are streamed once" % wbytes}
+                                              "traffic": measured_traffic("gemm_config1_bytes_per_call"),
+                                              "traffic_source": "committed rocprofv3 --pmc profile of this call (profiles/gemm_config1_rows16_hbm_traffic.md), "
+                                                                "NOT measured in this run",
+                                              "note": "algorithmic bytes 8*(N*K + M*K + 2*M*N) = %.0f per call: the weights are streamed once" % wbytes}
     for nm in ("softmax_q19_1x1024x128x1024", "softmax_q19_1x4096x128x1024", "silu_q23_1x512x18432", "silu_q23_1x8192x18432",
                "sigmoid_q23_1x512x18432", "sigmoid_q23_1x8192x18432", "rmsnorm_fused_500x7168", "rmsnorm_fused_16384x7168"):
         if nm in extra:
@@ -759,12 +762,13 @@ def run():
         os._exit(0)
 
 
-def measured_traffic():
-    """HBM bytes per launch of the config-4 GEMM kernel, from the committed rocprofv3 --pmc runs (FETCH_SIZE and
-    WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB copy): profiles/traffic.json."""
+def measured_traffic(key="gemm_config4_bytes_per_launch"):
+    """HBM bytes per launch of the config-4 GEMM kernel (or, with another key, per call of config 1), from the committed
+    rocprofv3 --pmc runs (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB copy):
+    profiles/traffic.json."""
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            return json.load(f).get("gemm_config4_bytes_per_launch")
+            return json.load(f).get(key)
     except (OSError, ValueError):
         return None
 
