@@ -105,6 +105,40 @@ def test_stale_guess_bmm(K, oracle, shape, w32):
     _stale_guess_rounds(K, _bmm(K, A, W, 29), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, 29), [A, W], pokes)
 
 
+@pytest.mark.parametrize("N", [256, 1024])            # A tracked inside the GEMM kernel / by the plane pre-pass
+@pytest.mark.parametrize("side", ["A", "B"])
+def test_tracked_digit_counts_at_the_borders(K, oracle, side, N):
+    """The kernels track the digit count an operand needs, not its extremes.  n balanced digits hold
+    [-0x80..80, 0x7F..7F] (n bytes each): one element exactly on a border must leave the digit count where it is, one
+    element past it must raise it by one, on either side of zero, whatever the other elements hold.  The digit count a
+    border value ends up with is compared with that of a plain value of the same width."""
+    rng = np.random.default_rng(700 + N)
+    M, Kd = 64, 256
+    keep = []                       # every operand at an address of its own: nothing remembered for it
+
+    def plan_with(value):
+        A = rand_i64(rng, (1, M, Kd), 12)
+        W = rand_i64(rng, (N, Kd), 12)
+        (A if side == "A" else W)[(0, 5, 7) if side == "A" else (N - 3, 9)] = value
+        dA, dW = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+        keep.extend((dA, dW))
+        for _ in range(3):          # the first call learns the range, the later ones run on it
+            C, R = K.int64_bmm_broadcast(dA, dW, 1, 1, 13)
+            torch.cuda.synchronize()        # (what a call has seen reaches the next one once its kernels are through)
+        Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 13)
+        assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+        return K.gemm_last_plan()
+    told_apart = 0
+    for n in (2, 3, 4, 5):
+        top, bottom = int("7F" * n, 16), -int("80" * n, 16)
+        fits, beyond = plan_with(1 << (8 * n - 9)), plan_with(1 << (8 * n - 1))       # n and n + 1 digits for certain
+        assert plan_with(top) == fits and plan_with(bottom) == fits, n
+        assert plan_with(top + 1) == beyond and plan_with(bottom - 1) == beyond, n
+        told_apart += fits != beyond
+    # (not every digit count has a kernel of its own: two digits run on three, five on six; some borders must show)
+    assert told_apart >= 2
+
+
 def test_stale_guess_whole_operands_widen(K, oracle):
     """both operands rewritten with full-range values under the same pointers (every tile and every k-step is wide)"""
     rng = np.random.default_rng(5)
