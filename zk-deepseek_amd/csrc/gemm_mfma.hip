@@ -50,6 +50,7 @@ static const Instance *instances(int *count)
         mfma_instances_rows32b(t);
         mfma_instances_rows32c(t);
         mfma_instances_rows32d(t);
+        mfma_instances_rows32e(t);
 #endif
         return t;
     }();

@@ -1046,5 +1046,6 @@ void mfma_instances_rows32(std::vector<Instance> &out);
 void mfma_instances_rows32b(std::vector<Instance> &out);
 void mfma_instances_rows32c(std::vector<Instance> &out);
 void mfma_instances_rows32d(std::vector<Instance> &out);
+void mfma_instances_rows32e(std::vector<Instance> &out);
 
 }  // namespace zk
