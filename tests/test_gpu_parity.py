@@ -450,6 +450,9 @@ def test_gemm_config4_full_size_sampled(K, oracle, path, full_range):
     C2, _ = K.int64_bmm_broadcast(Ad + A2, Wd, 1, 1, 0)
     assert torch.equal(C2, C0 + C1)
     assert torch.equal(C1, torch.roll(C0, 1, dims=1))
+    # shift 0 is the product modulo 2^64, and torch's CPU int64 matmul (the reference's CPU path) wraps the same way:
+    # a block of rows and columns is compared with it directly, full-range operands included
+    assert torch.equal(C0[0, 100:148, 4000:5024].cpu(), torch.matmul(A[0, 100:148], W[4000:5024].T))
 
 
 @pytest.mark.parametrize("seed", range(40 * SEEDS))
