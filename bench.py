@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
-Prints ONE JSON line.  `value` is the int64 GEMM throughput (Gmac/s) of BASELINE config 4
+Prints ONE JSON line.  `value` is the int64 GEMM throughput (Gmac/s) of benchmark config 4
 (512 x 7168 against W[18432,7168], config-1 operand ranges, shift 29) through the C ABI with operands
 resident in HBM; one step = one call of int64_64_bmm_broadcast_launcher.  The same line carries the
 other shapes the metric names (config-1 GEMM, full-range config 4, softmax / SiLU / sigmoid / RMSNorm
@@ -650,7 +650,7 @@ def run():
         einsum_leg("einsum_bsht_btc_bshc_1x1024x128xT1024_to_512", lambda: K.einsum_bsht_btc_bshc(pp, kvc, 23), Se * He * Se * Ce,
                    "einsum_bsht_btc_bshc", pp, kvc, 23)
         del pp, kvc
-        # config 3 as BASELINE states it: Q [1,1024,128,192] against K [1,1024,192] in one call, P.V with 128 columns
+        # config 3 as the benchmark set states it: Q [1,1024,128,192] against K [1,1024,192] in one call, P.V with 128 columns
         q3, k3 = rnd(16, 1, Se, He, 192), rnd(16, 1, Se, 192)
         einsum_leg("einsum_bshc_btc_bsht_config3_1x1024x128x192_T1024", lambda: K.einsum_bshc_btc_bsht(q3, k3, 21), Se * He * Se * 192,
                    "einsum_bshc_btc_bsht", q3, k3, 21)

@@ -1,4 +1,4 @@
-"""BASELINE configs 2, 3 and 5 as end-to-end chains: the same layer arithmetic (tests/harness.py, restating
+"""Benchmark configs 2, 3 and 5 as end-to-end chains: the same layer arithmetic (tests/harness.py, restating
 the glue of inference/model.py) runs on the HIP library and on the CPU oracle from the same seeded inputs,
 and every intermediate that leaves a kernel must agree bit for bit."""
 import numpy as np

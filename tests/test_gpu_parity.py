@@ -53,7 +53,7 @@ def _gemm_case(K, oracle, path, A, W, a_rs, b_rs, c):
 @pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("c", [0, 29])
 def test_gemm_config1_wkv_a(K, oracle, path, c):
-    """BASELINE config 1: Y[16,576] = X[16,7168] @ W[576,7168]^T, X in 2^20, W in 2^16, int64 W."""
+    """Benchmark config 1: Y[16,576] = X[16,7168] @ W[576,7168]^T, X in 2^20, W in 2^16, int64 W."""
     rng = np.random.default_rng(1000)
     A = rand_i64(rng, (1, 16, 7168), 20)
     W = rand_i64(rng, (576, 7168), 16)
@@ -418,7 +418,7 @@ def test_gemm_rejects_bad_arguments(K):
 @pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("full_range", [False, True])
 def test_gemm_config4_full_size_sampled(K, oracle, path, full_range):
-    """BASELINE config 4 at full size: 512 x 7168 against W[18432,7168].  The oracle checks a sample of rows and
+    """Benchmark config 4 at full size: 512 x 7168 against W[18432,7168].  The oracle checks a sample of rows and
     columns exactly; linearity in A (at shift 0, where the result is the wrapping int64 product) covers the rest."""
     if path == 1 and full_range:
         pytest.skip("one full-size VALU run is enough")
@@ -648,7 +648,7 @@ def test_softmax_unaligned_rows(K, oracle):
 
 
 def test_softmax_config3_full_size_properties(K, oracle):
-    """BASELINE config 3 softmax at full size [1,1024,128,1024]: exact on a sample of rows, invariants on all."""
+    """Benchmark config 3 softmax at full size [1,1024,128,1024]: exact on a sample of rows, invariants on all."""
     g = torch.Generator(device="cpu").manual_seed(3000)
     S, H, T = 1024, 128, 1024
     x = torch.randint(-(6 << 19), 6 << 19, (1, S, H, T), generator=g, dtype=torch.int64)
