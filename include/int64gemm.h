@@ -197,7 +197,9 @@ long zk_dump_flush(void);
  * int64_grouped_bmm_launcher: C[r][n] = (sum_k A[r][k] * B_e[n][k]) >> c_rescale (128-bit wrapping sum) and, when R
  *   is not null, R = that sum mod 2^c_rescale, for the rows r of expert e's segment; B_ptrs [groups] holds the
  *   experts' weight matrices ([N,K], int32 when b32 else int64).  Semantics of int64_64/32_bmm_broadcast_launcher
- *   per segment.  It waits for the device once per call (its digit check; see zk_gemm_guard_hits).
+ *   per segment.  The first call with a table of weights waits for the device once (its digit check); later calls
+ *   with that table do not wait: like the bmm launchers they run on remembered digit counts and are followed by a
+ *   guarded recomputation (see zk_gemm_guard_hits).
  * moe_combine: y[t][n] = sum_k (ye[sorted_pos[t][k]][n] * weights[t][k]) >> shift with wrapping products and sums
  *   (model.py:1379 with shift 23; floor, like torch's //). */
 void moe_dispatch(const int64_t *indices, int T, int K, int E, int *counts_scratch, int *seg, int *sorted_token,

@@ -84,7 +84,9 @@ struct GroupedDesc {
 bool gemm_gemv_grouped_launch(const GroupedDesc &d);
 
 // The grouped product on the 16-row MFMA tiles (see gemm_rows16_launch): one launch, no wait.  0 / 1 / -1 as there.
-int gemm_rows16_grouped(const GroupedDesc &d);
+// `guard`: a device word; when given, the launch's workgroups return at once unless it is non-zero (the fallback behind
+// a speculative launch of the 32-row kernels).
+int gemm_rows16_grouped(const GroupedDesc &d, const unsigned long long *guard = nullptr);
 
 // One launch of the 32-row-tile MFMA kernels over all groups.  Returns 0 when done, 1 when the operands need
 // more digits than those kernels are built for (nothing valid was written: the caller takes another route),

@@ -87,6 +87,7 @@ struct PendingRange {
     hipEvent_t ev = nullptr;
     unsigned long long *host = nullptr;      // pinned: [minA, maxA, minB, maxB, verdict]
     OperandKey key_a, key_b;
+    int nb_fixed = 0;                        // B came from prepared planes with this many digits (nothing of it was tracked)
     bool busy = false;
 };
 
@@ -188,6 +189,7 @@ static void drain_pending()
             const int64_t b_lo = (int64_t)(s.host[2] ^ kSignFlip), b_hi = (int64_t)(s.host[3] ^ kSignFlip);
             const int na_seen = limbs_needed((int64_t)(s.host[0] ^ kSignFlip), (int64_t)(s.host[1] ^ kSignFlip));
             if (b_lo <= b_hi) g_cache.store_pair(s.key_a, na_seen, s.key_b, limbs_needed(b_lo, b_hi));
+            else if (s.nb_fixed) g_cache.store_pair(s.key_a, na_seen, s.key_b, s.nb_fixed);      // (a grouped launch on prepared planes)
             else g_cache.store(s.key_a, na_seen);            // B came from prepared planes: nothing of it was tracked
             if (s.host[4]) g_cache.guard_hits++;
         }
@@ -737,13 +739,24 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
     }
     if (prep) { p.grp_b = prep->table; p.b_nsub = prep->nsub; p.b_ksteps = prep->ksteps; }
     int na = g_cache.lookup(key_a), nb = prep ? prep->nb : g_cache.lookup(key_b);
-    bool na_guessed = false;
+    bool na_guessed = false, informed = nb != 0;
     if (!na) {
         auto it = g_cache.partner_a.find(key_b);
         na = it != g_cache.partner_a.end() ? it->second : 5;
+        informed = informed && it != g_cache.partner_a.end();
         na_guessed = true;
     }
     if (!nb) nb = 5;
+    // Both digit counts come from what these weights met before: speculate, do not wait.  A guarded launch of the
+    // 16-row kernels follows on the stream (they guess nothing and take every operand); its workgroups return at once
+    // unless the verdict is bad, in which case they compute every output again.  What the kernels saw travels to pinned
+    // host memory behind an event and reaches the cache at a later call.  Otherwise (first sight of the weights, no
+    // free slot) the verdict is read back before the call returns, as it used to be for every grouped launch.
+    PendingRange *slot = nullptr;
+    if (informed && g_cache.pinned && !g_switches.sync_verdict) {
+        PendingRange &s = g_cache.pending[g_cache.pending_head];
+        if (!s.busy && s.ev) slot = &s;
+    }
 
     for (int attempt = 0; attempt < 3; attempt++) {
         const Instance *inst = nullptr;
@@ -790,8 +803,27 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
                 return -1;
             }
         }
-        const FoldArgs fold = make_fold(nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, nullptr);
+        const FoldArgs fold = make_fold(nullptr, 0, g_cache.wg, blocks, p.range, inst->na, inst->nb, slot ? slot->host : nullptr);
         range_fold_kernel<<<dim3((unsigned)fold.parts), 256, 0, 0>>>(fold);
+        if (slot) {
+            const int rc = gemm_rows16_grouped(d, p.range + 4);
+            if (rc < 0) return -1;
+            if (rc == 0) {
+                *limbs_a = inst->na;
+                *limbs_b = inst->nb;
+                if (hipEventRecord(slot->ev, 0) == hipSuccess) {
+                    slot->key_a = key_a;
+                    slot->key_b = key_b;
+                    slot->nb_fixed = prep ? prep->nb : 0;
+                    slot->busy = true;
+                    g_cache.pending_head = (g_cache.pending_head + 1) % kPendingSlots;
+                } else {
+                    (void)hipGetLastError();
+                }
+                return 0;
+            }
+            slot = nullptr;         // the 16-row kernels do not take this product: wait for the verdict after all
+        }
         int64_t r[4];
         if (!read_range(p.range, r)) { set_error(kLaunchFailure, "grouped gemm: range readback failed"); return -1; }
         const int need_a = limbs_needed(r[0], r[1]), need_b = prep ? prep->nb : limbs_needed(r[2], r[3]);

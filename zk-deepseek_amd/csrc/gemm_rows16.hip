@@ -42,6 +42,8 @@ struct Rows16Params {
     // grouped mode: rows of A and C form one segment per group, every group has its own B (see GroupedDesc)
     const int *grp_seg, *grp_tiles, *grp_ntiles;
     const void *const *grp_b;
+    const unsigned long long *guard;     // when set: do nothing unless this word is non-zero
+    unsigned items;                      // work items of the launch (the grid may be smaller: workgroups walk them)
 };
 
 constexpr int kR16Fast = 9;              // diagonals the accumulators hold: digit pairs up to (5, 5)
@@ -218,7 +220,7 @@ __device__ __forceinline__ void step_fast(const RawFrag<false> &fa_raw, const Ra
 }
 
 template <bool B32, bool GRP>
-__global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Params p)
+__device__ __forceinline__ void rows16_item(const Rows16Params &p, unsigned item)
 {
     typedef R16Shape<B32> S;
     constexpr int CT = S::kColTiles, LPT = S::kLoadsPerTile;
@@ -230,7 +232,6 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
     const unsigned ring_a_lds = (unsigned)(uintptr_t)ring_a, ring_w_lds = (unsigned)(uintptr_t)ring_w;   // LDS byte addresses
 
     // workgroup -> (batch or 32-row tile half, four column groups, K slice); the wavefronts take the column groups
-    unsigned item = blockIdx.x;                                     // (the host keeps the count below 2^31)
     const int cg4 = (p.col_groups + kR16Waves - 1) / kR16Waves;
     int slice = 0;
     if (p.nslices > 1) { slice = (int)(item % (unsigned)p.nslices); item /= (unsigned)p.nslices; }
@@ -475,6 +476,20 @@ __global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Param
         for (int r = 0; r < 4; r++) slot[(ct * 4 + r) * 64 + lane] = sums[ct][r];
 }
 
+// One workgroup per item (a tile of 16 rows, four column groups, a slice of K), or, behind a guard word, a grid of one
+// workgroup per compute unit that walks the items: such a launch is the fallback behind a speculative launch of the
+// 32-row kernels and almost always has nothing to do, which a grid of ten thousand workgroups of 128 KB of LDS each
+// takes 60 us to find out.
+template <bool B32, bool GRP>
+__global__ __launch_bounds__(64 * kR16Waves) void gemm_rows16_kernel(Rows16Params p)
+{
+    if (p.guard && *p.guard == 0) return;            // (the same for every thread of the launch)
+    for (unsigned item = blockIdx.x; item < p.items; item += gridDim.x) {
+        rows16_item<B32, GRP>(p, item);
+        if (item + gridDim.x < p.items) __syncthreads();           // (the rings are used again)
+    }
+}
+
 // Adds the slots of every output tile, applies rounding term and shift, stores C and R.  Four threads share an output
 // (each adds every fourth slice with all its loads under way at once, then the four meet through shuffles): the launch
 // is a chain of one load latency, not of one per slice.
@@ -609,10 +624,13 @@ static bool r16_fill(const GemmDesc &d, Rows16Params &p)
 
 typedef void (*Rows16Kernel)(Rows16Params);
 
-static int r16_run(Rows16Kernel fn, const Rows16Params &p, long blocks)
+static int r16_run(Rows16Kernel fn, const Rows16Params &params, long blocks)
 {
     if (blocks > 0x7FFFFFF0L) return 1;
     constexpr int lds = kR16LdsBytes;
+    Rows16Params p = params;
+    p.items = (unsigned)blocks;
+    if (p.guard && blocks > r16_cus()) blocks = r16_cus();
     static const void *raised[4] = {};
     bool seen = false;
     for (const void *f : raised) seen = seen || f == (const void *)fn;
@@ -675,7 +693,7 @@ int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_sl
     return 0;
 }
 
-int gemm_rows16_grouped(const GroupedDesc &d)
+int gemm_rows16_grouped(const GroupedDesc &d, const unsigned long long *guard)
 {
     if (d.K < 0 || d.N < 1 || d.rows < 1 || d.groups < 1) return 1;
     const int cols = d.b32 ? R16Shape<true>::kCols : R16Shape<false>::kCols;
@@ -687,6 +705,7 @@ int gemm_rows16_grouped(const GroupedDesc &d)
     p.col_groups = (d.N + cols - 1) / cols;
     p.nslices = 1;
     p.grp_seg = d.seg; p.grp_tiles = d.tiles; p.grp_ntiles = d.ntiles; p.grp_b = d.B;
+    p.guard = guard;
     // the grid covers the worst case of the tile table (the host never learns the segment sizes): rows / 32 + groups
     // tiles of 32 rows, two halves each
     const long blocks = ((long)d.rows / 32 + d.groups) * 2 * ((p.col_groups + kR16Waves - 1) / kR16Waves);
