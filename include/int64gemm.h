@@ -111,7 +111,7 @@ void zk_clear_error(void);
 size_t zk_workspace_bytes(void);
 size_t zk_prepared_weights_bytes(void);
 void zk_release_workspace(void);
-/* Reads the diagnosis switches ZK_GEMM_SYNC, ZK_NO_TAIL_SPLIT, ZK_B_ROWS_MIN_MACS and ZK_ROWS16_MAX_WEIGHTS from the
+/* Reads the diagnosis switches ZK_GEMM_SYNC, ZK_NO_TAIL_SPLIT, ZK_B_ROWS_MIN_MACS, ZK_ROWS16_MAX_WEIGHTS and ZK_SKINNY_MAX_M from the
  * environment again (they are read once when the library is loaded, not per call). */
 void zk_reload_env(void);
 

@@ -136,9 +136,13 @@ static RangeCache g_cache;
 
 // Diagnosis switches, read from the environment once when the library is loaded (and again on zk_reload_env):
 // ZK_GEMM_SYNC: every call waits for its own digit verdict; ZK_NO_TAIL_SPLIT: no split-K; ZK_B_ROWS_MIN_MACS: product
-// size from which a small n-contiguous int64 B is rewritten with contiguous rows first.
-struct Switches { bool sync_verdict, no_tail_split; double b_rows_min_macs; };
+// size from which a small n-contiguous int64 B is rewritten with contiguous rows first; ZK_SKINNY_MAX_M: rows up to
+// which the 32-row tiles are used.
+struct Switches { bool sync_verdict, no_tail_split; double b_rows_min_macs; int skinny_max_m; };
 constexpr long kBRowsMinMacs = 1L << 32;
+// Rows up to which a product runs on the 32-row tiles (two of them from 33 rows on): measured against the 128-row tiles,
+// 48 rows x [1536,7168] int32 34.1 against 38.1 us, 64 x [2048,7168] int64 37.6-39.4 against 41.2, 128 rows 56.8 against 45.1.
+constexpr int kSkinnyMaxRows = 64;
 static Switches read_switches()
 {
     Switches s;
@@ -146,6 +150,8 @@ static Switches read_switches()
     s.no_tail_split = getenv("ZK_NO_TAIL_SPLIT") != nullptr;
     const char *m = getenv("ZK_B_ROWS_MIN_MACS");
     s.b_rows_min_macs = m ? atof(m) : (double)kBRowsMinMacs;
+    const char *sk = getenv("ZK_SKINNY_MAX_M");
+    s.skinny_max_m = sk ? atoi(sk) : kSkinnyMaxRows;
     return s;
 }
 static Switches g_switches = read_switches();
@@ -539,14 +545,14 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         // the stored bits are [shift, shift + 64) of the sum (the remainder lies below them)
         const int need_diag = (d.shift + 64 + 7) / 8;
         // (the kernels that read planes never see B's element type: they are the int64 forms)
-        const Instance *inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0 && !prep, true, need_diag, prep ? prep->nb : 0, prep ? kB64FlyBPlanes : -1) : nullptr;
+        const Instance *inst = d.M <= g_switches.skinny_max_m ? pick_instance(na, nb, d.b32 != 0 && !prep, true, need_diag, prep ? prep->nb : 0, prep ? kB64FlyBPlanes : -1) : nullptr;
         if (!inst) inst = pick_instance(na, nb, d.b32 != 0 && !prep, false, need_diag, prep ? prep->nb : 0, prep ? kB64PlanesBoth : -1);
         if (!inst && prep) {
             // no kernel with exactly the planes' digit count covers A: this call splits the original B like any other
             // (nb, the planes' count, covers B)
             prep = nullptr;
             p.B = d.B;
-            inst = d.M <= 32 ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
+            inst = d.M <= g_switches.skinny_max_m ? pick_instance(na, nb, d.b32 != 0, true, need_diag) : nullptr;
             if (!inst) inst = pick_instance(na, nb, d.b32 != 0, false, need_diag);
         }
         if (!inst) return kDeclined;
