@@ -21,7 +21,9 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libzkoracle.so")
+# ZK_ORACLE_LIB names another build of zk_oracle.c to load instead: the mutant test uses it to show that the pin
+# suite rejects perturbed copies of the oracle
+_SO = os.environ.get("ZK_ORACLE_LIB") or os.path.join(_HERE, "libzkoracle.so")
 
 
 def build(force=False):

@@ -238,7 +238,7 @@ def test_gemm_one_or_two_rows(K, oracle, M, w32):
 @pytest.mark.parametrize("M", [1, 3, 8, 15, 16])
 def test_gemm_up_to_16_rows(K, oracle, M, w32):
     """the 16-row MFMA tiles (every wavefront on its own, digit counts taken from each step's data): one K slice and
-    several (partial sums added atomically, the last slice finishes), ragged N and K, batches, every digit path from
+    several (every slice writes its partial sums into a slot of its own, a second launch adds the slots), ragged N and K, batches, every digit path from
     (3,3) to (5,5), operands beyond five digits (the wavefronts that meet them recompute on the vector ALU), widths that
     change from step to step, every shift class, with and without remainder"""
     rng = np.random.default_rng(160 + M + w32)
@@ -301,9 +301,10 @@ def test_gemm_up_to_16_rows(K, oracle, M, w32):
     K.lib.zk_gemm_set_path(0)
 
 
-def test_gemm_split_k_scratch_is_left_zeroed(K, oracle):
-    """several K slices per output tile add into scratch that the last slice leaves zeroed: calls of different shapes one
-    after the other, asynchronously, must not see each other's partial sums"""
+def test_gemm_split_k_slots_of_an_earlier_call_do_not_show_through(K, oracle):
+    """the K slices of a call write partial sums into slots that the library keeps between calls, and nothing clears
+    them: calls of different shapes one after the other, asynchronously (a larger one before a smaller one, the same
+    one twice), must each add up their own slots only"""
     rng = np.random.default_rng(170)
     K.lib.zk_gemm_set_path(2)
     shapes = [(16, 7168, 576), (5, 4096, 64), (16, 7168, 576), (9, 2048, 1000), (3, 8192, 33)]
@@ -634,6 +635,44 @@ def test_softmax_hostile_inputs(K, oracle, fn):
         torch.cuda.synchronize()
         Ce, _ = getattr(oracle, fn)(x, table)
         assert np.array_equal(host(C), Ce)
+
+
+def test_softmax_and_activation_hand_worked_literals(K):
+    """the results worked by hand from the reference's source (the steps are written out in test_oracle_pins.py:
+    softmax q19 :700-740 and q21 :624-657 of inference/int64_gemm.cu, sigmoid/SiLU q23 :932-946 and q25 :804-818),
+    asked of the device library directly: no oracle in between"""
+    def smx(fn, row):
+        R = dev(np.array(row, np.int64).reshape(1, 1, 1, -1))
+        C = torch.empty_like(R)
+        getattr(K, fn)(R, C)
+        return host(C).ravel().tolist()
+
+    def act(fn, vals):
+        R = dev(np.array(vals, np.int64).reshape(1, 1, -1))
+        C = torch.empty_like(R)
+        getattr(K, fn)(R, C)
+        return host(C).ravel().tolist()
+
+    assert smx("softmax_q19", [0, -(1 << 19)]) == [383193, 141094]
+    assert smx("softmax_q19", [0, 0, 0, 0, -(1 << 42), -(1 << 42), -(1 << 42), -(1 << 42)]) == [1 << 17] * 4 + [0] * 4
+    assert smx("softmax_q21", [0, -11356, -2924304]) == [933750, 931225, 232177]     # rounded exponent, rounded quotient
+    assert smx("softmax_q21", [0, -(1 << 42)]) == [1 << 21, 0]
+    assert smx("softmax_q21", [0, -6096986655889]) == [1 << 21, 0]                   # the product wraps: the clip decides
+    assert act("sigmoid_q23", [-(1 << 23), 3, -22713, 0]) == [2257517, 4199982, 1 << 22, 1 << 22]
+    assert act("silu_q23", [-(1 << 23), -22713, 0]) == [-2257517, -11357, 0]
+    assert act("sigmoid_q25", [-90852, 181705, 3, -407108648]) == [16754503, 16822642, 16799929, 180]
+    assert act("silu_q25", [-90852, 181705]) == [-45365, 91098]
+    # the same values in the middle of a long tensor, where the table kernels and the vector loads take them
+    vals = np.zeros(70000, np.int64)
+    vals[[5, 4099, 65537]] = [-90852, 181705, -407108648]
+    out = np.array(act("sigmoid_q25", vals))
+    assert out[[5, 4099, 65537]].tolist() == [16754503, 16822642, 180] and (np.delete(out, [5, 4099, 65537]) == 1 << 24).all()
+    vals[[5, 4099, 65537]] = [-22713, -(1 << 23), 3]
+    out = np.array(act("sigmoid_q23", vals))
+    assert out[[5, 4099, 65537]].tolist() == [1 << 22, 2257517, 4199982]
+    row = np.full(1024, -(1 << 42), np.int64)
+    row[[0, 500, 1023]] = [0, -11356, -2924304]
+    assert np.array(smx("softmax_q21", row))[[0, 500, 1023]].tolist() == [933750, 931225, 232177]
 
 
 def test_softmax_unaligned_rows(K, oracle):

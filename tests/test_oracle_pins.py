@@ -151,6 +151,21 @@ def test_einsum_rounding_term_is_half_the_shift_count(oracle):
     assert oracle.einsum_bshc_btc_bsht(a, b, 23)[0, 0, 0, 0] == 0
 
 
+def test_each_einsum_has_its_own_rounding_term(oracle):
+    """one product of 1 * v per output, so the sum is v: the first three einsums add rescale/2 = 11 before >> 23
+    (inference/int64_gemm.cu:401, :442, :483), the fourth adds nothing (:525)"""
+    v = (1 << 23) - 11
+    for below in (0, 1):
+        a = np.full((1, 1, 1, 1), v - below, np.int64)
+        assert oracle.einsum_bshd_hdc_bshc(a, np.ones((1, 1, 1), np.int32), 23)[0, 0, 0, 0] == 1 - below
+        assert oracle.einsum_bshc_btc_bsht(a, np.ones((1, 1, 1), np.int64), 23)[0, 0, 0, 0] == 1 - below
+        assert oracle.einsum_bsht_btc_bshc(a, np.ones((1, 1, 1), np.int64), 23)[0, 0, 0, 0] == 1 - below
+        assert oracle.einsum_bshc_hdc_bshd(a, np.ones((1, 1, 1), np.int32), 23)[0, 0, 0, 0] == 0
+    a = np.full((1, 1, 1, 1), 1 << 23, np.int64)
+    assert oracle.einsum_bshc_hdc_bshd(a, np.ones((1, 1, 1), np.int32), 23)[0, 0, 0, 0] == 1
+    assert oracle.einsum_bshc_hdc_bshd(a - 1, np.ones((1, 1, 1), np.int32), 23)[0, 0, 0, 0] == 0
+
+
 # ------------------------------------------------------------------- RoPE ---
 def test_rope_identity_and_bigint(oracle):
     rng = np.random.default_rng(5)
@@ -192,6 +207,15 @@ def test_rms_stat_is_isqrt(oracle, bits):
         q = acc // 7168
         assert rms[m] == math.isqrt(q)
         assert int(rms[m]) ** 2 <= q < (int(rms[m]) + 1) ** 2        # zk/src/index.ts:989-996
+
+
+def test_rms_stat_adds_eps_before_dividing(oracle):
+    """inference/kernel.py:477-494: (eps + sum a^2) // dim.  Row [1,1,1,0] with dim 4: (1 + 3) // 4 = 1 -> rms 1; a
+    statistic that drops eps gets 3 // 4 = 0.  Row of four 3s with dim 4: (1 + 36) // 4 = 9 -> 3; dividing by dim - 1 or
+    rounding up would not."""
+    A = np.array([[1, 1, 1, 0], [3, 3, 3, 3], [2, 2, 2, 1]], np.int64)
+    assert oracle.rms_stat(A, 1, 4).tolist() == [1, 3, 1]            # (1 + 13) // 4 = 3 -> isqrt 1
+    assert oracle.rms_stat(A, 3, 4).tolist() == [1, 3, 2]            # (3 + 13) // 4 = 4 -> 2
 
 
 @pytest.mark.parametrize("w32", [True, False])
@@ -255,6 +279,61 @@ def test_softmax_q19_single_element_steps(oracle):
     assert abs(w[0, 0, 0, 1] / 2 ** 19 - math.exp(-1)) < 2e-3
 
 
+def test_softmax_q21_hand_steps_rounded_exponent_and_rounded_quotient(oracle):
+    """Worked by hand from inference/int64_gemm.cu:624-657 at inputs where each rounding decides the result.
+
+    Row [0, -11356, -2924304] (max 0, so d = x).  LOG2E_Q21 = 3025551, 2^21 = 2097152, 2^20 = 1048576.
+    d = -11356:   d*L = -34358157156.  -16384*2^21 = -34359738368 < d*L < -16383*2^21 = -34357641216, and
+                  d*L + 2^20 = -34357108580 > -16383*2^21, so y = -16383 (:634; WITHOUT the + 2^20 it is -16384).
+                  -y = 16383: k = 0, f = 16383, f >> 13 = 1 (:636-641; 16384 >> 13 would be 2), w = LUT[1].
+    d = -2924304: d*L = -8847630891504 = -4218879.2.. * 2^21, + 2^20 -> y = -4218879 (floor alone: -4218880).
+                  -y = 4218879 = 2*2^21 + 24575: k = 2, f = 24575, f >> 13 = 2 (24576 >> 13 would be 3), w = LUT[2] >> 2.
+    LUT[i] = floor(2^21 * 2^(-i/256)) (:672-680): LUT[1] = 2091481, LUT[2] = 2085826 -- the reference holds no copy of
+    this table, so the two literals are checked below by the exact inequality v^256 <= 2^(256*21 - i) < (v+1)^256.
+    w = [2097152, 2091481, 521456], sumW = 4710089, sumW/2 = 2355044 (:656-657):
+      (2097152*2^21 + 2355044) / 4710089 = 933750      (without the + sumW/2: 933750)
+      (2091481*2^21 + 2355044) / 4710089 = 931225      (931225)
+      ( 521456*2^21 + 2355044) / 4710089 = 232177      (232176: the rounding of the quotient decides)"""
+    for i, v in ((1, 2091481), (2, 2085826)):
+        assert v ** 256 <= 1 << (256 * 21 - i) < (v + 1) ** 256
+    assert oracle.softmax_init_q21()[:3].tolist() == [2097152, 2091481, 2085826]
+    x = np.array([0, -11356, -2924304], np.int64).reshape(1, 1, 1, 3)
+    C, w = oracle.softmax_q21(x)
+    assert w[0, 0, 0].tolist() == [2097152, 2091481, 521456]
+    assert C[0, 0, 0].tolist() == [933750, 931225, 232177]
+    # the same arithmetic in exact integers, so that the literals above are not only the oracle's word
+    assert -16384 * 2097152 < -11356 * 3025551 < -16383 * 2097152 < -11356 * 3025551 + 1048576
+    assert -4218880 * 2097152 < -2924304 * 3025551 < -4218879 * 2097152 < -2924304 * 3025551 + 1048576
+    assert 4218879 == 2 * 2097152 + 24575 and 2 * 8192 <= 24575 < 3 * 8192 and 2085826 // 4 == 521456
+    s = 2097152 + 2091481 + 521456
+    assert 232177 * s <= 521456 * 2097152 + s // 2 < 232178 * s and 521456 * 2097152 < 232177 * s
+
+
+def test_softmax_clips_decide_for_distances_beyond_the_products_width(oracle):
+    """The clips (inference/int64_gemm.cu:706 `d > 64<<19`, :627 `d < -(64<<21)`) change nothing for moderate distances
+    (there k >= 64 or the table entry shifted by k >= 22 is 0 anyway: at d = 2^25 resp. -2^27 exactly both branches give
+    0, so `>` against `>=` cannot be told apart by any input), but they are what keeps a masked element at 0 once the
+    product leaves its width: q21 multiplies in 64 bits (:634), and -2^42 * 3025551 = -1.33e19 wraps to a positive y,
+    which without the clip indexes the table with a negative k; q19's y is the low 64 bits of a 128-bit product (:713),
+    negative for d = 2^63."""
+    x = np.array([0, -(1 << 42)], np.int64).reshape(1, 1, 1, 2)           # the causal mask value, inference/model.py:1555
+    C, w = oracle.softmax_q21(x)
+    assert w[0, 0, 0].tolist() == [1 << 21, 0] and C[0, 0, 0].tolist() == [1 << 21, 0]
+    for lo in (-(1 << 62), -(1 << 62) - 12345, -(1 << 63) + (1 << 62) - 99):
+        x = np.array([1 << 62, lo, (1 << 62) - 1], np.int64).reshape(1, 1, 1, 3)
+        C, w = oracle.softmax_q19(x)
+        assert w[0, 0, 0, :2].tolist() == [1 << 19, 0] and C[0, 0, 0, 1] == 0
+    x = np.array([(1 << 62), -(1 << 62), -(1 << 61)], np.int64).reshape(1, 1, 1, 3)
+    C, w = oracle.softmax_q21(x)
+    assert w[0, 0, 0].tolist() == [1 << 21, 0, 0]
+    # d = -ceil(2^64 / 3025551) = -6096986655889 (about 1.4 times the mask value): d * L = -(2^64 + 2068223) wraps to
+    # -2068223, whose y = -1 would index the table at k = 0 and give w = 2^21, as much as the maximum itself
+    assert 6096986655889 * 3025551 == (1 << 64) + 2068223
+    x = np.array([0, -6096986655889], np.int64).reshape(1, 1, 1, 2)
+    C, w = oracle.softmax_q21(x)
+    assert w[0, 0, 0].tolist() == [1 << 21, 0] and C[0, 0, 0].tolist() == [1 << 21, 0]
+
+
 # ------------------------------------------------------------- activations ---
 @pytest.mark.parametrize("Q", [23, 25])
 def test_sigmoid_silu_special_values_and_float(oracle, Q):
@@ -286,11 +365,46 @@ def test_sigmoid_q23_hand_steps(oracle):
     x = np.array([-(1 << 23)], np.int64)
     assert oracle.sigmoid_q23(x)[0] == 2257517
     assert oracle.silu_q23(x)[0] == (-(1 << 23) * 2257517) >> 23 == -2257517
+    # x = -22713: (-x) * L = 274877336739 < 2^38 = 274877906944, so y = 32767, table cell 0, u = 2^23, q = 2^46 / 2^24.
+    # Negating AFTER the shift (as q25 does, :804) gives -floor(-32767.9..) = 32768: cell 1, q = 4188625.
+    assert 22713 * 12102203 == 274877336739 < 1 << 38
+    x = np.array([-22713], np.int64)
+    assert oracle.sigmoid_q23(x)[0] == 1 << 22
+    assert oracle.silu_q23(x)[0] == -11357                  # floor(-22713 * 2^22 / 2^23) = floor(-11356.5)
     # q23 negates before the shift, q25 after: they differ in rounding for positive inputs
     # x = 3, q23: y = (-3 * 12102203) >> 23 = -5, k = -1, f = 2^23 - 5, index 255; q25: y = -((3 * 48408813) >> 25) = -4
     x = np.array([3], np.int64)
     assert oracle.sigmoid_q23(x)[0] == 4199982
     assert oracle.sigmoid_q25(x)[0] == 16799929
+
+
+def test_sigmoid_silu_q25_hand_steps_negation_after_the_shift(oracle):
+    """Worked by hand from inference/int64_gemm.cu:804-818: y = -int64((r * 48408813) >> 25) floors BEFORE negating
+    (q23 negates first, :932), which moves y by one whenever the product is not a multiple of 2^25.
+
+    r = -90852: r*L = -4398037478676, and -2^42 = -4398046511104 < r*L < -131071 * 2^25 = -4398012956672, so the
+    arithmetic shift gives -131072 and y = 131072 = 2^17: k = 0, f = 2^17, f >> 17 = 1, u = t = LUT25[1] = 33645407.
+    (Negating first: (90852*L) >> 25 = 131071, f >> 17 = 0, t = 2^25, q = 2^50 / 2^26 = 16777216.)
+    q = 2^50 / (2^25 + 33645407) = 1125899906842624 / 67199839 = 16754503;  SiLU = (r*q) >> 25 = floor(-45364.2) = -45365.
+    r = 181705: r*L = 8796123366165 = 262144.9.. * 2^25, so y = -262144 (negating first: -262145): k = -1,
+    f = 2^25 - 262144 = 33292288, f >> 17 = 254 (33292287 >> 17 = 253), u = LUT25[254] >> 1 = 66746437 >> 1 = 33373218,
+    q = 2^50 / (2^25 + 33373218) = 16822642; SiLU = (181705 * 16822642) >> 25 = 91098.
+    LUT25[i] = floor(2^25 * 2^(i/256)) (:832-839); the reference holds no copy, so the literals are checked exactly."""
+    for i, v in ((1, 33645407), (254, 66746437)):
+        assert v ** 256 <= 1 << (256 * 25 + i) < (v + 1) ** 256
+    lut = oracle.silu_init_q25().tolist()
+    assert lut[0] == 1 << 25 and lut[1] == 33645407 and lut[254] == 66746437
+    assert -(1 << 42) < -90852 * 48408813 < -131071 * (1 << 25)
+    assert 16754503 * 67199839 <= 1 << 50 < 16754504 * 67199839
+    assert 262144 * (1 << 25) < 181705 * 48408813 < 262145 * (1 << 25)
+    assert 16822642 * ((1 << 25) + 33373218) <= 1 << 50 < 16822643 * ((1 << 25) + 33373218)
+    x = np.array([-90852, 181705], np.int64)
+    assert oracle.sigmoid_q25(x).tolist() == [16754503, 16822642]
+    assert oracle.silu_q25(x).tolist() == [-45365, 91098]
+    assert -45365 * (1 << 25) <= -90852 * 16754503 < -45364 * (1 << 25)
+    assert 91098 * (1 << 25) <= 181705 * 16822642 < 91099 * (1 << 25)
+    # the same two inputs through q23's order of operations land one table cell away (what :932 against :804 means)
+    assert oracle.sigmoid_q25(np.array([-407108648], np.int64))[0] == 180          # (r*L) >> 25 = -587333632, k = 17, cell 129
 
 
 # -------------------------------------------------------------------- float -> fixed converters ---
