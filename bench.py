@@ -249,7 +249,13 @@ def run():
         roofline = {"bound": "valu", "achieved": achieved, "peak": None, "unit": "Tmac/s", "frac": None,
                     "traffic": None, "note": "VALU 64-bit multiply-add path; no published peak"}
 
+    launch_floor_us = None
     if legs & {"extra", "small"}:
+        # what two dependent, nearly empty launches cost back to back (the shape of a split-K call: a streaming kernel
+        # and a finishing kernel), measured on this device: the part of config 1's time that no kernel can remove
+        launch_floor_us = K.lib.zk_probe_launch_pair_us(252, 200)
+        K._check("launch pair probe")
+        extra["launch_pair_252_workgroups_us"] = launch_floor_us
         # the GEMMs smaller than the device ("small" alone: the legs a kernel trace of them needs)
         # config 1 (M=16): weight-bandwidth bound
         g1 = torch.Generator(device="cpu").manual_seed(1000)
@@ -304,6 +310,69 @@ def run():
         K.lib.zk_gemm_set_path(1 if path == 2 else 2)
         extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1, samples, "gemm_config4_other_path", host=(A_h, W_h))
         K.lib.zk_gemm_set_path(0)
+
+        # Calls on operands the library has not seen.  The reference's driver builds every layer anew on the device for
+        # every position (inference/generate.py:227-238) and loads each routed expert from disk when it is hit
+        # (inference/model.py:1362-1363), so in an unchanged drop-in the weight pointers of most calls are new, or are
+        # recycled addresses that hold other contents than last time.  Wall clock of ONE call from before the call to
+        # after a device synchronisation (so a readback that blocks the host is inside), next to the same single call
+        # on warm operands: (a) freshly allocated A and W at addresses never passed before; (b) a known address whose
+        # contents were overwritten in place with wider values (W from 17 to 31 bits) since the library last saw it.
+        def one_call_ms(fn):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            t_ret = time.perf_counter()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3, (t_ret - t0) * 1e3
+
+        def cold_leg(name, Mc, Kc, Nc, shift):
+            gc_ = torch.Generator(device="cuda").manual_seed(4100 + Mc)
+            keep = []                       # everything stays allocated: no address comes back
+            mk = lambda lo, hi, *shape: torch.randint(lo, hi, shape, generator=gc_, dtype=torch.int64, device="cuda")
+            Cc = torch.empty((1, Mc, Nc), dtype=torch.int64, device="cuda")
+            Rc = torch.empty_like(Cc)
+            fn64 = K.lib.int64_64_bmm_broadcast_launcher
+
+            def call(Ax, Wx):
+                fn64(Ax.data_ptr(), Wx.data_ptr(), Cc.data_ptr(), Rc.data_ptr(), 1, 1, shift, 1, Mc, Kc, Nc)
+
+            res = {}
+            firsts, blocked = [], []
+            for rep in range(3):
+                Ax, Wx = mk(-(1 << 20), 1 << 20, 1, Mc, Kc), mk(-(1 << 16), 1 << 16, Nc, Kc)
+                keep += [Ax, Wx]
+                ms, ret = one_call_ms(lambda: call(Ax, Wx))
+                firsts.append(ms)
+                blocked.append(ret)
+            K._check(name)
+            res["first_call_new_addresses_ms"] = sorted(firsts)[1]
+            res["first_call_host_blocked_ms"] = sorted(blocked)[1]
+            Ax, Wx = keep[-2], keep[-1]
+            for _ in range(3):
+                call(Ax, Wx)
+            warm = sorted(one_call_ms(lambda: call(Ax, Wx)) for _ in range(5))[2]
+            res["warm_single_call_ms"], res["warm_host_blocked_ms"] = warm
+            # the same addresses, wider contents written in place behind the library's back
+            Wx.copy_(mk(-(1 << 30), 1 << 30, Nc, Kc))
+            hits0 = K.lib.zk_gemm_guard_hits()
+            ms, ret = one_call_ms(lambda: call(Ax, Wx))
+            res["recycled_address_wider_contents_ms"] = ms
+            res["recycled_address_host_blocked_ms"] = ret
+            samples.append(gemm_sample(name + "_recycled", Ax, Wx, Cc, Rc, shift))
+            ms2, _ = one_call_ms(lambda: call(Ax, Wx))
+            res["call_after_that_ms"] = ms2
+            res["guarded_recomputations"] = int(K.lib.zk_gemm_guard_hits() - hits0)
+            K._check(name)
+            res["first_over_warm"] = res["first_call_new_addresses_ms"] / res["warm_single_call_ms"]
+            res["recycled_over_warm"] = res["recycled_address_wider_contents_ms"] / res["warm_single_call_ms"]
+            extra[name] = res
+            del keep
+
+        cold_leg("cold_gemm_config4_512x7168x18432", 512, 7168, 18432, 29)
+        cold_leg("cold_gemm_config2_w1_128x7168x2048", 128, 7168, 2048, 16)
+        cold_leg("cold_gemm_config1_16x7168x576", 16, 7168, 576, 29)
+        torch.cuda.empty_cache()
 
         # memory-bound kernels, 16 algorithmic bytes per element
         K.softmax_init_q19()
@@ -711,8 +780,11 @@ def run():
     else:
         verified["other_legs"] = "not compared in this run (--no-cpu skips the CPU leg that holds the comparisons)"
 
-    # roofline of the HBM-bound shapes the metric names, from this run's HIP-event timings
+    # Rooflines of the other shapes the metric names, from this run's HIP-event timings.  They live INSIDE "roofline" as
+    # flat numbers (the record a driver keeps of this line may hold known keys only and drop nested objects), and once
+    # more, with their notes, under roofline["others"].
     others = {}
+    flat = {}
     if "gemm_config1_16x7168x576" in extra:
         e = extra["gemm_config1_16x7168x576"]
         wbytes = 8.0 * (576 * 7168 + 16 * 7168 + 2 * 16 * 576)
@@ -722,30 +794,70 @@ def run():
                                               "traffic_source": "committed rocprofv3 --pmc profile of this call (profiles/gemm_config1_rows16_hbm_traffic.md), "
                                                                 "NOT measured in this run",
                                               "note": "algorithmic bytes 8*(N*K + M*K + 2*M*N) = %.0f per call: the weights are streamed once" % wbytes}
+        flat["gemm_config1_us"] = e["ms"] * 1e3
+        flat["gemm_config1_gmacs"] = e["gmacs"]
+        flat["gemm_config1_GBps"] = gbs
+        flat["gemm_config1_frac_hbm"] = gbs / HBM_PEAK_GBS
+        flat["gemm_config1_traffic"] = measured_traffic("gemm_config1_bytes_per_call")
+        if launch_floor_us is not None:
+            # what two dependent launches cost on this device whatever they compute, plus the weights at the HBM peak
+            floor_us = launch_floor_us + wbytes / (HBM_PEAK_GBS * 1e9) * 1e6
+            flat["gemm_config1_two_launch_floor_us"] = launch_floor_us
+            flat["gemm_config1_frac_of_launch_floor_plus_hbm"] = floor_us / (e["ms"] * 1e3)
+    for nm, short in (("gemm_config2_w1_128x7168x2048", "gemm_config2_w1_us"), ("gemm_config2_w2_128x2048x7168", "gemm_config2_w2_us")):
+        if nm in extra:
+            flat[short] = extra[nm]["ms"] * 1e3
     for nm in ("softmax_q19_1x1024x128x1024", "softmax_q19_1x4096x128x1024", "silu_q23_1x512x18432", "silu_q23_1x8192x18432",
                "sigmoid_q23_1x512x18432", "sigmoid_q23_1x8192x18432", "rmsnorm_fused_500x7168", "rmsnorm_fused_16384x7168"):
         if nm in extra:
             e = extra[nm]
             others[nm] = {"bound": "hbm", "achieved": e["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": e["frac_hbm_peak"],
                           "traffic": None, "note": "16 algorithmic bytes per element (8 read + 8 written)"}
+            flat[nm + "_GBps"] = e["GBps"]
+            flat[nm + "_frac_hbm"] = e["frac_hbm_peak"]
+    for nm in ("moe_experts_int32_256tok_top8_of_256", "moe_experts_config5_256tok_top8_of_256"):
+        if nm in extra:
+            flat[nm + "_frac_hbm"] = extra[nm]["frac_hbm_peak"]
+    roofline.update(flat)
+    roofline["others"] = others
+    cold = {}
+    for nm, short in (("cold_gemm_config4_512x7168x18432", "config4"), ("cold_gemm_config2_w1_128x7168x2048", "config2_w1"),
+                      ("cold_gemm_config1_16x7168x576", "config1")):
+        if nm in extra:
+            e = extra[nm]
+            cold[short + "_first_call_ms"] = e["first_call_new_addresses_ms"]
+            cold[short + "_warm_call_ms"] = e["warm_single_call_ms"]
+            cold[short + "_recycled_wider_ms"] = e["recycled_address_wider_contents_ms"]
+    all_checked = "cpu" in legs
 
+    config = {"workload": "config4: int64 GEMM Y[512,18432] = X[512,7168] @ W[18432,7168]^T, int64 W, "
+                          "X in [-2^20,2^20), W in [-2^16,2^16), c_rescale=29, C and R written",
+              "path": {1: "valu", 2: "mfma_i8"}.get(path, "?"), "limbs_a": la, "limbs_b": lb,
+              "kernel_ms_hip_events": kern_ms,
+              "verified": bool(all_checked),
+              "untimed_calls_before_the_timed_steps": untimed_calls,
+              "untimed_calls_note": "warmup steps asked for plus calls keeping the device busy %d ms (idle clocks)" % SPIN_UP_MS}
+    if "gemm_config1_us" in flat:
+        config["gemm_config1_us"] = flat["gemm_config1_us"]
+    config.update(cold)
+    # the figures a reader wants first, once more at the very end of the line (a record that keeps only the tail of the
+    # output still holds them)
+    summary = {"value_gmacs": value, "ms_per_step": ms_per_step, "roofline_frac": roofline.get("frac"), "verified": bool(all_checked)}
+    summary.update({k: v for k, v in flat.items() if k.endswith(("_us", "_frac_hbm"))})
+    summary.update(cold)
+    if cpu_baseline:
+        summary["cpu_baseline_gmacs"] = cpu_baseline.get("value")
     out = {
         "metric": "int64 GEMM Gmac/s @7168x576 & 18432x7168 + softmax/SiLU HBM GB/s, 1 MI355X",
         "value": value, "unit": "Gmac/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int64", "data": "synthetic",
-        "config": {"workload": "config4: int64 GEMM Y[512,18432] = X[512,7168] @ W[18432,7168]^T, int64 W, "
-                               "X in [-2^20,2^20), W in [-2^16,2^16), c_rescale=29, C and R written",
-                   "path": {1: "valu", 2: "mfma_i8"}.get(path, "?"), "limbs_a": la, "limbs_b": lb,
-                   "kernel_ms_hip_events": kern_ms,
-                   "untimed_calls_before_the_timed_steps": untimed_calls,
-                   "untimed_calls_note": "the %d warmup steps asked for plus the calls it takes to keep the device busy "
-                                         "for %d ms (an idle MI355X needs that long to reach its clocks)" % (args.warmup, SPIN_UP_MS)},
+        "config": config,
         "roofline": roofline,
-        "roofline_others": others,
         "cpu_baseline": cpu_baseline,
         "verified": verified,
         "extra": extra,
+        "summary": summary,
     }
     # everything is released and flushed before the line is printed, so that nothing lingers behind it
     K.dump_flush()

@@ -210,8 +210,10 @@ void int64_grouped_bmm_launcher(const int64_t *A, const void *const *B_ptrs, int
                                 int rows, int K, int N);
 void moe_combine(const int64_t *ye, const int64_t *weights, const int *sorted_pos, int64_t *y, int T, int K, int N, int shift);
 
-/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc): the product of int64_64/32_bmm_broadcast_launcher (b32 != 0: B
+/* No counterpart in the reference.  For callers that cannot allocate device memory (tight serving loops,
+ * harnesses that forbid hipMalloc; NOT for capture into a HIP graph as it stands: its two kernels are launched on the
+ * null stream, which a capturing stream does not record, and the first call on a device also looks up the array's
+ * address and sets a kernel attribute): the product of int64_64/32_bmm_broadcast_launcher (b32 != 0: B
  * holds int32) for up to 16 rows, a_rescale fixed at 1 and b_rescale a positive power of two, on kernels whose scratch
  * (the partial sums of a K split) is a static 8 MB array in device memory instead of a buffer the library allocates.
  * It allocates nothing, frees nothing and waits for nothing.  Limits: M <= 16 and Bdim * M * N <= 2^20 outputs; anything
@@ -263,6 +265,10 @@ int zk_gemm_last_prepared(void);
  * instead of zeros (the device is power managed and the rate depends on how the operand bits toggle).
  * Allocates 4 bytes for the duration of the call and waits for its kernels. */
 double zk_probe_mfma_i8_tops(int with_lds, int random_data, int steps);
+/* Microseconds per repetition of two dependent, nearly empty launches back to back on the null stream (`workgroups`
+ * workgroups store 16 bytes each, a second kernel reads them): what the launches alone cost a call that is made of a
+ * streaming kernel and a finishing kernel.  A measurement aid for bench.py; not needed for inference. */
+double zk_probe_launch_pair_us(int workgroups, int reps);
 
 /* HIP-event stopwatch on the null stream (the stream every entry point launches on). */
 void zk_timer_start(void);

@@ -81,7 +81,9 @@ def test_no_alloc_entry_point_allocates_nothing_and_rejects_what_it_cannot_take(
     Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, 29)
     assert np.array_equal(C.cpu().numpy(), Ce) and np.array_equal(R.cpu().numpy(), Re)
     # beyond the limits: a clear error, nothing launched
-    for args in ((1, 29, 1, 17, 7168, 576), (1, 29, 1, 16, 64, (1 << 16) + 1), (3, 29, 1, 16, 7168, 576), (1, 64, 1, 16, 7168, 576)):
+    # (the last two: output counts whose product leaves 64 bits -- 2^30 * 16 * 2^30 wraps to 0 -- and one that wraps into the limit)
+    for args in ((1, 29, 1, 17, 7168, 576), (1, 29, 1, 16, 64, (1 << 16) + 1), (3, 29, 1, 16, 7168, 576), (1, 64, 1, 16, 7168, 576),
+                 (1, 29, 1 << 30, 16, 64, 1 << 30), (1, 29, (1 << 31) - 1, 16, 64, (1 << 31) - 1)):
         K.lib.int64_bmm_broadcast_noalloc(dA.data_ptr(), dW.data_ptr(), 0, C.data_ptr(), R.data_ptr(), *args)
         assert K.lib.zk_last_error() in (1, 3), args
         K.lib.zk_clear_error()

@@ -699,6 +699,7 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             if (hipEventRecord(slot->ev, 0) == hipSuccess) {
                 slot->key_a = key_a;
                 slot->key_b = key_b;
+                slot->nb_fixed = prep ? prep->nb : 0;       // (the slots are shared with the grouped launches, which set it too)
                 slot->busy = true;
                 g_cache.pending_head = (g_cache.pending_head + 1) % kPendingSlots;
             } else {

@@ -27,6 +27,7 @@
 #include "gemm_mfma_kernels.h"
 
 #include <cstdlib>
+#include <mutex>
 
 namespace zk {
 
@@ -69,7 +70,11 @@ constexpr int kR16LdsBytes = kR16StagesA * 8192 + kR16Waves * kR16StagesW * 8192
 __device__ __forceinline__ void lds_dma16(const void *gptr, unsigned lds_base)
 {
     // (the base is the same in every lane, but derived from the wavefront's number, which the compiler holds in a vector register)
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr) : "memory");
+    // M0 is put back as it was: the compiler does not see the statement write it (the register cannot be named as
+    // clobbered) and may be keeping a value of its own there across the statement.
+    unsigned saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr) : "memory");
 }
 
 template <int N>
@@ -545,18 +550,29 @@ namespace zk {
 static unsigned long long *g_r16_acc = nullptr;
 static size_t g_r16_slots = 0;
 static int g_r16_cus = 0;
+static std::mutex g_r16_mu;              // host threads take turns in the launchers below (the scratch may be regrown, the attribute list filled)
 
 constexpr size_t kR16SlotBytes = 8 * 64 * 16;
 constexpr int kNoAllocMaxRows = 16;                        // limits of int64_bmm_broadcast_noalloc
 constexpr long kNoAllocMaxOutputs = 1L << 20;
 
-size_t gemm_rows16_workspace_bytes() { return g_r16_slots * kR16SlotBytes; }
-
-void gemm_rows16_release_workspace()
+static void r16_release_locked()
 {
     if (g_r16_acc) (void)hipFree(g_r16_acc);
     g_r16_acc = nullptr;
     g_r16_slots = 0;
+}
+
+size_t gemm_rows16_workspace_bytes()
+{
+    std::lock_guard<std::mutex> lock(g_r16_mu);
+    return g_r16_slots * kR16SlotBytes;
+}
+
+void gemm_rows16_release_workspace()
+{
+    std::lock_guard<std::mutex> lock(g_r16_mu);
+    r16_release_locked();
 }
 
 static int r16_cus()
@@ -576,7 +592,7 @@ static int r16_scratch(size_t slots)
     // the old buffer may still be in use by launches under way: the stream is drained first (this happens a few times
     // in a process, while the largest launch is still growing)
     if (g_r16_slots && hipStreamSynchronize(0) != hipSuccess) { set_error(kLaunchFailure, "gemm: cannot wait for the stream"); return -1; }
-    gemm_rows16_release_workspace();
+    r16_release_locked();
     if (hipMalloc(&g_r16_acc, slots * kR16SlotBytes) != hipSuccess) {
         (void)hipGetLastError();
         g_r16_acc = nullptr;
@@ -666,6 +682,7 @@ int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_sl
     Rows16Params p;
     if (!r16_fill(d, p)) return 1;
     if (!acc && (long)d.N * d.K > g_r16_max_weights) return 1;
+    std::lock_guard<std::mutex> lock(g_r16_mu);
     const long tiles = (long)d.G * p.row_tiles * p.col_groups;
     const long wg_tiles = (long)d.G * p.row_tiles * ((p.col_groups + kR16Waves - 1) / kR16Waves);
     if (tiles > (1L << 24)) return 1;
@@ -696,6 +713,7 @@ int gemm_rows16_launch(const GemmDesc &d, unsigned long long *acc, size_t max_sl
 int gemm_rows16_grouped(const GroupedDesc &d, const unsigned long long *guard)
 {
     if (d.K < 0 || d.N < 1 || d.rows < 1 || d.groups < 1) return 1;
+    std::lock_guard<std::mutex> lock(g_r16_mu);
     const int cols = d.b32 ? R16Shape<true>::kCols : R16Shape<false>::kCols;
     Rows16Params p = {};
     p.A = d.A; p.B = nullptr; p.C = d.C; p.R = d.R;
@@ -715,7 +733,7 @@ int gemm_rows16_grouped(const GroupedDesc &d, const unsigned long long *guard)
 }  // namespace zk
 
 // ---- the entry point that allocates nothing -----------------------------------------------------------------
-// Callers under HIP graph capture, tight serving loops and harnesses that forbid it cannot call hipMalloc.  For them the
+// Tight serving loops and harnesses that forbid it cannot call hipMalloc.  For them the
 // scratch of the split-K launches is a file-scope device array: each GPU the library runs on holds its own copy, at its
 // own address, until the process ends.  The array's name is a host-side stand-in, not a device address: its address on
 // the current device is looked up once per device and that pointer is what the kernels get.
@@ -761,11 +779,12 @@ extern "C" void int64_bmm_broadcast_noalloc(const int64_t *A, const void *B, int
         return;
     }
     if (M > kNoAllocMaxRows) { set_error(kUnsupportedSize, "%s: %d rows, at most %d", name, M, kNoAllocMaxRows); return; }
-    if ((long)Bdim * M * N > kNoAllocMaxOutputs) {
-        set_error(kUnsupportedSize, "%s: %ld outputs, at most %ld", name, (long)Bdim * M * N, kNoAllocMaxOutputs);
+    if (Bdim == 0 || M == 0 || N == 0) return;
+    // (each factor on its own first: the product of three ints can leave 64 bits)
+    if (Bdim > kNoAllocMaxOutputs || N > kNoAllocMaxOutputs || (long)Bdim * M > kNoAllocMaxOutputs || (long)Bdim * M * N > kNoAllocMaxOutputs) {
+        set_error(kUnsupportedSize, "%s: %d x %d x %d outputs, at most %ld", name, Bdim, M, N, kNoAllocMaxOutputs);
         return;
     }
-    if ((long)Bdim * M * N == 0) return;
     if (!A || !B || !C) { set_error(kBadArgument, "%s: null pointer", name); return; }
     unsigned long long *ptr = noalloc_scratch(name);
     if (!ptr) return;

@@ -58,7 +58,50 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int steps, int random_d
     if (s == 0x7f3a91c5 && steps < 0) sink[0] = s;       // never true: keeps the accumulators alive
 }
 
+// The smallest thing a call made of two dependent launches can be: every workgroup of the first kernel stores 16 bytes,
+// every thread group of the second loads them and stores one word.  What this pair costs per repetition, back to back on
+// the null stream, is what the launches themselves cost a split-K call (one kernel that streams, one that adds up).
+__global__ __launch_bounds__(256) void probe_pair_first(unsigned long long *buf)
+{
+    if (threadIdx.x == 0) {
+        buf[2 * blockIdx.x] = blockIdx.x;
+        buf[2 * blockIdx.x + 1] = ~(unsigned long long)blockIdx.x;
+    }
+}
+
+__global__ __launch_bounds__(256) void probe_pair_second(const unsigned long long *buf, unsigned long long *out, int n)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = buf[2 * i] + buf[2 * i + 1];
+}
+
 }  // namespace zk
+
+extern "C" double zk_probe_launch_pair_us(int workgroups, int reps)
+{
+    if (workgroups <= 0 || workgroups > 65536 || reps <= 0) { zk::set_error(zk::kBadArgument, "zk_probe_launch_pair_us: bad argument"); return 0.0; }
+    unsigned long long *buf = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    double us = 0.0;
+    if (hipMalloc(&buf, (size_t)workgroups * 3 * sizeof(unsigned long long)) == hipSuccess && hipEventCreate(&t0) == hipSuccess &&
+        hipEventCreate(&t1) == hipSuccess) {
+        auto pair = [&] {
+            zk::probe_pair_first<<<dim3((unsigned)workgroups), dim3(256), 0, 0>>>(buf);
+            zk::probe_pair_second<<<dim3((unsigned)((workgroups + 255) / 256)), dim3(256), 0, 0>>>(buf, buf + 2 * (size_t)workgroups, workgroups);
+        };
+        for (int r = 0; r < 10; r++) pair();
+        (void)hipEventRecord(t0, 0);
+        for (int r = 0; r < reps; r++) pair();
+        (void)hipEventRecord(t1, 0);
+        float ms = 0.f;
+        if (hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess && ms > 0.f) us = (double)ms * 1e3 / reps;
+    }
+    if (hipGetLastError() != hipSuccess || us == 0.0) zk::set_error(zk::kLaunchFailure, "zk_probe_launch_pair_us: measurement failed");
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    if (buf) (void)hipFree(buf);
+    return us;
+}
 
 extern "C" double zk_probe_mfma_i8_tops(int with_lds, int random_data, int steps)
 {

@@ -88,6 +88,8 @@ lib.zk_dump_host.argtypes = [ctypes.c_char_p, _vp, ctypes.c_size_t]
 lib.zk_dump_flush.restype = ctypes.c_long
 lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
+lib.zk_probe_launch_pair_us.argtypes = [_ci, _ci]
+lib.zk_probe_launch_pair_us.restype = ctypes.c_double
 lib.zk_workspace_bytes.restype = ctypes.c_size_t
 lib.zk_prepared_weights_bytes.restype = ctypes.c_size_t
 
