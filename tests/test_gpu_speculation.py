@@ -153,6 +153,78 @@ def test_stale_guess_whole_operands_widen(K, oracle):
     _stale_guess_rounds(K, _bmm(K, A, W, 7), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, 7), [A, W], [widen])
 
 
+@pytest.mark.parametrize("fallback", ["mfma", "valu"])
+@pytest.mark.parametrize("w32", [False, True])
+def test_stale_guess_both_kinds_of_guarded_launch(K, oracle, fallback, w32, monkeypatch):
+    """the launch behind a speculative product is the widest MFMA instance, one workgroup per compute unit walking the
+    tiles (row-major B: nine digits for int64, five for int32), or the vector-ALU tiles (ZK_VALU_FALLBACK, and whatever
+    the MFMA form does not take).  Shapes with fewer tiles than compute units and with several tiles per workgroup,
+    ragged edges, batches, a remainder or none, every element wide or a single one."""
+    import os
+    if fallback == "valu":
+        monkeypatch.setenv("ZK_VALU_FALLBACK", "1")
+    else:
+        monkeypatch.delenv("ZK_VALU_FALLBACK", raising=False)
+    K.lib.zk_reload_env()
+    try:
+        rng = np.random.default_rng(900 + w32)
+        for Bd, M, Kd, N, c in ((1, 40, 300, 90, 29), (2, 130, 520, 1300, 0), (1, 700, 96, 1500, 33)):
+            A = Operand(rand_i64(rng, (Bd, M, Kd), 20))
+            W = Operand(rand_i32(rng, (N, Kd), 16) if w32 else rand_i64(rng, (N, Kd), 16))
+
+            def widen():
+                A.h[...] = rand_i64(rng, A.h.shape, 63)
+                W.h[...] = rand_i32(rng, W.h.shape, 31) if w32 else rand_i64(rng, W.h.shape, 63)
+                A.d.copy_(torch.from_numpy(A.h))
+                W.d.copy_(torch.from_numpy(W.h))
+            pokes = [widen, lambda: A.poke((Bd - 1, M - 1, Kd - 1), -(1 << 62)), lambda: W.poke((N - 1, 0), (1 << 30) if w32 else (1 << 62))]
+            _stale_guess_rounds(K, _bmm(K, A, W, c), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, c), [A, W], pokes)
+        # without a remainder
+        A = Operand(rand_i64(rng, (1, 70, 200), 20))
+        W = Operand(rand_i32(rng, (300, 200), 16) if w32 else rand_i64(rng, (300, 200), 16))
+        _stale_guess_rounds(K, lambda: (K.int64_bmm_broadcast(A.d, W.d, 1, 1, 17, want_remainder=False)[0],),
+                            lambda: (oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, 17)[0],), [A, W],
+                            [lambda: A.poke((0, 3, 5), 1 << 61)])
+    finally:
+        monkeypatch.delenv("ZK_VALU_FALLBACK", raising=False)
+        K.lib.zk_reload_env()
+
+
+def test_stale_guess_long_k_falls_back_to_the_vector_alu(K, oracle):
+    """nine digits over K = 16384 do not fit the int32 accumulators of one pass (the guarded MFMA form does not split K):
+    the vector-ALU tiles stand behind such a product"""
+    rng = np.random.default_rng(950)
+    A = Operand(rand_i64(rng, (1, 40, 16384), 20))
+    W = Operand(rand_i64(rng, (70, 16384), 16))
+    _stale_guess_rounds(K, _bmm(K, A, W, 29), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, 29), [A, W],
+                        [lambda: A.poke((0, 39, 16383), -(1 << 62)), lambda: W.poke((5, 7), 1 << 62)])
+
+
+def test_operands_at_new_addresses_run_on_the_digits_of_their_shape(K, oracle):
+    """a product below 2^34 MACs whose operands lie at addresses never seen takes the digits of the last operands of the
+    same shapes and does not wait; wider values than those are caught by the guarded launch like any stale guess"""
+    rng = np.random.default_rng(960)
+    keep = []
+    M, Kd, N = 72, 264, 136            # (a shape no other test uses)
+    def fresh(bits_a, bits_w):
+        a, w = rand_i64(rng, (1, M, Kd), bits_a), rand_i64(rng, (N, Kd), bits_w)
+        keep.extend((torch.from_numpy(a).cuda(), torch.from_numpy(w).cuda()))
+        C, R = K.int64_bmm_broadcast(keep[-2], keep[-1], 1, 1, 19)
+        plan = K.gemm_last_plan()
+        Ce, Re = oracle.int64_bmm_broadcast(a, w, 1, 1, 19)
+        assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+        torch.cuda.synchronize()
+        return plan
+    assert fresh(20, 16) == (2, 3, 3)            # first of its shape: sampled
+    hits = K.lib.zk_gemm_guard_hits()
+    assert fresh(20, 16) == (2, 3, 3)
+    assert K.lib.zk_gemm_guard_hits() == hits
+    assert fresh(45, 40) == (2, 3, 3)            # runs on the shape's digits, is caught, and teaches the shape
+    assert K.lib.zk_gemm_guard_hits() == hits + 1
+    plan = fresh(45, 40)
+    assert plan[1] >= 6 and plan[2] >= 6 and K.lib.zk_gemm_guard_hits() == hits + 1
+
+
 def test_stale_guess_fresh_activations_known_weights(K, oracle):
     """what a model does in every layer: a NEW activation tensor against weights seen before.  The digits of A are
     guessed from the activations last multiplied with those weights; wider ones must be caught."""

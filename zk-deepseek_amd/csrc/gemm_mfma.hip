@@ -97,6 +97,7 @@ struct RangeCache {
     std::mutex mu;
     std::map<OperandKey, int> limbs;         // operand -> digits its values needed when last seen
     std::map<OperandKey, int> partner_a;     // B operand -> digits of the A operand it was last multiplied with
+    std::map<std::tuple<long, long, int>, int> by_shape;      // (rows, K, element size) -> digits of the last operand of that shape, wherever it lay
     unsigned long long *dev = nullptr;       // [minA, maxA, minB, maxB, verdict]
     unsigned char *planes = nullptr;         // digit planes of A, grown on demand, kept for the process lifetime
     size_t planes_bytes = 0;
@@ -122,6 +123,15 @@ struct RangeCache {
     {
         if (limbs.size() > 4096) limbs.clear();
         limbs[k] = n;
+        if (by_shape.size() > 4096) by_shape.clear();
+        by_shape[std::make_tuple(std::get<1>(k), std::get<2>(k), std::get<3>(k))] = n;
+    }
+    // An operand at an address never seen (or seen with another shape): what the last operand of its shape needed.  The
+    // weights of one kind of projection need the same digits in every layer, and so do the activations that meet them.
+    int lookup_shape(const OperandKey &k)
+    {
+        auto it = by_shape.find(std::make_tuple(std::get<1>(k), std::get<2>(k), std::get<3>(k)));
+        return it == by_shape.end() ? 0 : it->second;
     }
     void store_pair(const OperandKey &ka, int na, const OperandKey &kb, int nb)
     {
@@ -135,11 +145,13 @@ struct RangeCache {
 static RangeCache g_cache;
 
 // Diagnosis switches, read from the environment once when the library is loaded (and again on zk_reload_env):
-// ZK_GEMM_SYNC: every call waits for its own digit verdict; ZK_NO_TAIL_SPLIT: no split-K; ZK_B_ROWS_MIN_MACS: product
+// ZK_GEMM_SYNC: every call waits for its own digit verdict; ZK_NO_TAIL_SPLIT: no split-K; ZK_VALU_FALLBACK: the guarded launch
+// behind a speculative one is always the vector-ALU kernel; ZK_B_ROWS_MIN_MACS: product
 // size from which a small n-contiguous int64 B is rewritten with contiguous rows first; ZK_SKINNY_MAX_M: rows up to
 // which the 32-row tiles are used.
-struct Switches { bool sync_verdict, no_tail_split; double b_rows_min_macs; int skinny_max_m; };
+struct Switches { bool sync_verdict, no_tail_split, valu_fallback; double b_rows_min_macs; int skinny_max_m; };
 constexpr long kBRowsMinMacs = 1L << 32;
+constexpr double kShapeGuessMaxMacs = 17179869184.0;        // 2^34: about 0.15 ms on the matrix pipe
 // Rows up to which a product runs on the 32-row tiles (two of them from 33 rows on): measured against the 128-row tiles,
 // 48 rows x [1536,7168] int32 34.1 against 38.1 us, 64 x [2048,7168] int64 37.6-39.4 against 41.2, 128 rows 56.8 against 45.1.
 constexpr int kSkinnyMaxRows = 64;
@@ -148,6 +160,7 @@ static Switches read_switches()
     Switches s;
     s.sync_verdict = getenv("ZK_GEMM_SYNC") != nullptr;
     s.no_tail_split = getenv("ZK_NO_TAIL_SPLIT") != nullptr;
+    s.valu_fallback = getenv("ZK_VALU_FALLBACK") != nullptr;
     const char *m = getenv("ZK_B_ROWS_MIN_MACS");
     s.b_rows_min_macs = m ? atof(m) : (double)kBRowsMinMacs;
     const char *sk = getenv("ZK_SKINNY_MAX_M");
@@ -467,6 +480,63 @@ __global__ __launch_bounds__(256) void b_rows_kernel(const int64_t *__restrict__
 // 16-byte loads and take A from digit planes (measured at S = T = 1024, 128 heads: 1.67 -> 1.45 ms, the rewrite 9 us).
 constexpr long kBRowsMaxElements = 8L << 20;         // 64 MB
 
+// The launch behind a speculative one: it does nothing unless the verdict word says that the digit counts did not cover
+// the operands, and then computes every output again.  Row-major B without a divisor: the widest MFMA instance (nine
+// digits hold every int64, five every int32; config 4 with stale three-digit guesses: 4 ms where the vector-ALU tiles
+// take 35), one workgroup per compute unit walking the tiles.  Everything else, and a K beyond what its int32
+// accumulators take in one piece: the vector-ALU tiles.
+static Outcome launch_guarded_fallback(const GemmDesc &d, const MfmaParams &spec, int b_shift)
+{
+    // (an n-contiguous B that the speculative launch read through its row-major copy is read through that copy here too)
+    const bool b_copied = spec.B == (const void *)g_cache.b_rows && g_cache.b_rows != nullptr;
+    const bool row_major = b_copied || !(d.ldbn == 1 && d.ldbk != 1);
+    const Instance *wide = (row_major && b_shift == 0 && !g_switches.valu_fallback) ? pick_instance(9, d.b32 ? 5 : 9, d.b32 != 0, false, 16) : nullptr;
+    MfmaKernel fn = wide ? wide->guarded[d.b32 ? 1 : 0] : nullptr;
+    if (fn) {
+        const long pairs = wide->na < wide->nb ? wide->na : wide->nb;
+        const int ksteps = ((d.K + 32 * wide->kk - 1) / (32 * wide->kk)) * wide->kk;
+        if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) fn = nullptr;
+    }
+    MfmaParams q = spec;
+    if (fn) {
+        // the caller's operands, not digit planes
+        q.A = d.A; q.lda = d.lda; q.sA = d.sA;
+        if (!b_copied) { q.B = d.B; q.ldbn = d.ldbn; q.ldbk = d.ldbk; q.sB = d.sB; }
+        q.a_planes = nullptr; q.a_msub = 0; q.a_ksteps = 0; q.b_nsub = 0; q.b_ksteps = 0;
+        q.tiles_m = (d.M + wide->bm - 1) / wide->bm;
+        q.tiles_n = (d.N + wide->bn - 1) / wide->bn;
+        const long total = (long)q.tiles_m * q.tiles_n * d.G;
+        if (total > 0x7FFFFFFFL / 8) fn = nullptr;
+        else {
+            q.main_tiles = (int)total; q.split = 1; q.tail_xcd = 0; q.partials = nullptr; q.part64 = 0; q.n_fastest = 0;
+            q.guard = spec.range + 4;
+            q.walk_blocks = (int)total;
+            // (the range slots of the speculative launch have been folded by now: the fallback's tracking may overwrite them)
+            const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)total * 4, "range slots");
+            if (got == kFailed) return kFailed;
+            if (got == kDeclined) fn = nullptr;
+            q.wg_range = g_cache.wg;
+        }
+    }
+    if (!fn) {
+        gemm_valu_launch(d, spec.range + 4);
+        return kDone;
+    }
+    const size_t lds = 2 * (size_t)wide->kk * ((wide->bm / 32) * wide->na + (wide->bn / 32) * wide->nb) * 1024 + 9 * 1024 + 16;
+    static std::set<const void *> lds_raised;
+    if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
+        if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+            set_error(kLaunchFailure, "gemm: cannot raise the LDS limit to %zu bytes", lds);
+            return kFailed;
+        }
+        lds_raised.insert((const void *)fn);
+    }
+    const long grid = q.walk_blocks < g_cache.cus ? q.walk_blocks : g_cache.cus;
+    fn<<<dim3((unsigned)grid), dim3((unsigned)wide->threads), lds, 0>>>(q);
+    if (hipGetLastError() != hipSuccess) { set_error(kLaunchFailure, "gemm: guarded MFMA launch failed"); return kFailed; }
+    return kDone;
+}
+
 int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
 {
     // Operand divisors: a power of two on B is folded into the digit split of the 32-row kernels (the head projection
@@ -523,9 +593,18 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         auto it = g_cache.partner_a.find(key_b);
         if (it != g_cache.partner_a.end()) na = it->second;
     }
-    // Operands seen before: speculate, do not wait.  Otherwise sample them and check the verdict before returning.
+    // Operands at addresses never seen: for products below kShapeGuessMaxMacs the digits of the last operands of the
+    // same shapes stand in (a wrong guess costs such a product less than the wait for a sample would: the reference's
+    // driver builds every layer anew, generate.py:227-238, so most of its calls come with new or recycled addresses);
+    // larger products, and shapes never seen, are sampled, which waits for the stream once.
+    if ((!na || !nb) && (double)d.G * d.M * d.N * d.K < kShapeGuessMaxMacs) {
+        if (!na) na = g_cache.lookup_shape(key_a);
+        if (!nb) nb = g_cache.lookup_shape(key_b);
+    }
+    // No call waits for its verdict (unless no slot is free for the range to travel in, or ZK_GEMM_SYNC asks for it): a
+    // guarded launch behind the product redoes it with digits that cover everything if the verdict is bad.
     PendingRange *slot = nullptr;
-    if (na && nb && g_cache.pinned && !g_switches.sync_verdict) {
+    if (g_cache.pinned && !g_switches.sync_verdict) {
         PendingRange &s = g_cache.pending[g_cache.pending_head];
         if (!s.busy && s.ev) slot = &s;
     }
@@ -646,7 +725,9 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             else if (k_over) return kDeclined;
         }
         const long blocks = (long)p.main_tiles + (total - p.main_tiles) * p.split;
-        if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;
+        // (room for the guarded fallback's 64 x 64 tiles as well, so that it never has to regrow the buffer)
+        const long fb_blocks = (long)((d.M + 63) / 64) * ((d.N + 63) / 64) * d.G;
+        if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)(blocks > fb_blocks ? blocks : fb_blocks) * 4, "range slots")) return got;
         p.wg_range = g_cache.wg;
 
         long plane_wgs = 0;
@@ -694,8 +775,8 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         *limbs_a = inst->na;
         *limbs_b = inst->nb;
         if (slot) {
-            // no waiting: the vector-ALU kernel redoes the product if the verdict is bad, the range follows later
-            gemm_valu_launch(d, p.range + 4);
+            // no waiting: a guarded launch redoes the product if the verdict is bad, the range follows later
+            if (const Outcome got = launch_guarded_fallback(d, p, b_shift)) return got;
             if (hipEventRecord(slot->ev, 0) == hipSuccess) {
                 slot->key_a = key_a;
                 slot->key_b = key_b;

@@ -52,6 +52,10 @@ struct MfmaParams {
     const void *const *grp_b;       // [groups] B of every group
     int b_shift;                    // BRS kernels: every element of B is divided by 2^b_shift first, truncating toward zero
     int finish_rq;                  // workgroups per tile of the finishing kernel (4 or 16)
+    // guarded launches (the fallback behind a speculative launch): the kernel does nothing unless *guard is non-zero, and
+    // its workgroups, one per compute unit, walk the `walk_blocks` workgroup ids of an ordinary launch
+    const unsigned long long *guard;
+    int walk_blocks;
 };
 
 constexpr unsigned long long kSignFlip = 0x8000000000000000ull;
@@ -437,9 +441,10 @@ __host__ __device__ constexpr int kept_pairs_before(int na, int nb, int d, int i
 // outputs that are never stored), only a final partial k-step uses guarded loads, and every thread walks its
 // own row pointers.  Loads of step s+1 are issued first, the MFMAs of the step's leading depths give them time
 // to land, and the MFMAs of the last depth are interleaved with the digit split of the loaded data.
+// (the body of the kernels below: `block` is the workgroup id of an ordinary launch, one tile or one slice of a split tile)
 template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false, int DMAX = 16,
           bool BPL = false>
-__global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
+__device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int block)
 {
     constexpr int T = 64 * WVM * WVN;
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 32 * KK, OCTS = BK / 8;
@@ -460,14 +465,14 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     // ids are regrouped to give each XCD a contiguous run of tiles; within a run the tile-row index moves
     // fastest, so the workgroups that share a B tile sit on the same L2.
     const int per_batch = p.tiles_m * p.tiles_n;
-    int lin = blockIdx.x, sidx = 0, nsplit = 1;
+    int lin = block, sidx = 0, nsplit = 1;
     int tail_tile = 0, g = 0, tn, tm, m0, m_lim = p.M;
     const void *b_base = p.B;
     if (GRP) {
         const int mt = lin / p.tiles_n;
         if (mt >= *p.grp_ntiles) {                 // the grid covers the worst case: nothing to do, an empty range
             if (tid == 0) {
-                unsigned long long *slot = p.wg_range + 4 * (long)blockIdx.x;
+                unsigned long long *slot = p.wg_range + 4 * (long)block;
                 slot[0] = ~0ull; slot[1] = 0ull; slot[2] = ~0ull; slot[3] = 0ull;
             }
             return;
@@ -830,7 +835,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
         }
     }
     if (tid == 0) {
-        unsigned long long *slot = p.wg_range + 4 * (long)blockIdx.x;
+        unsigned long long *slot = p.wg_range + 4 * (long)block;
         slot[0] = (unsigned long long)ra.lo ^ kSignFlip;
         slot[1] = (unsigned long long)ra.hi ^ kSignFlip;
         slot[2] = (unsigned long long)rb.lo ^ kSignFlip;
@@ -900,6 +905,27 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
     const bool edge = m0 + BM > m_lim || n0 + BN > p.N;
     if (p.R) { if (edge) store_tile(std::true_type(), std::true_type()); else store_tile(std::false_type(), std::true_type()); }
     else { if (edge) store_tile(std::true_type(), std::false_type()); else store_tile(std::false_type(), std::false_type()); }
+}
+
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, bool BKM, bool APL, bool GRP = false, bool BRS = false, int DMAX = 16,
+          bool BPL = false>
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
+{
+    gemm_mfma_block<NA, NB, WVM, WVN, WM, WN, KK, B32, BKM, APL, GRP, BRS, DMAX, BPL>(p, (int)blockIdx.x);
+}
+
+// The same product behind a guard word: nothing happens unless *p.guard is non-zero (the verdict of the speculative launch
+// in front of it: its digit counts did not cover the operands), and then the grid, one workgroup per compute unit, walks
+// the workgroup ids of an ordinary launch.  A guarded launch almost always finds nothing to do, and thousands of
+// workgroups with 80 KB of LDS each would take tens of microseconds to find that out.
+template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, int DMAX = 16>
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_guarded_kernel(MfmaParams p)
+{
+    if (__atomic_load_n(p.guard, __ATOMIC_RELAXED) == 0) return;            // (the same for every thread of the launch)
+    for (int block = (int)blockIdx.x; block < p.walk_blocks; block += (int)gridDim.x) {
+        gemm_mfma_block<NA, NB, WVM, WVN, WM, WN, KK, B32, false, false, false, false, DMAX, false>(p, block);
+        __syncthreads();            // (the LDS stages and the range words in them are used again)
+    }
 }
 
 // Adds the `split` partial sums of every tail tile, applies the rounding term and the shift, and stores C and R.
@@ -975,6 +1001,7 @@ struct Instance {
     MfmaKernel fn[kVariants];
     PlanesKernel planes[2];      // [b32]: the owned-k pattern follows the element size of B
     FinishKernel finish;         // adds up the partial sums of split tail tiles (and folds the ranges)
+    MfmaKernel guarded[2];       // [b32]: the guarded form for row-major B, A split on the fly (the widest instances only)
 };
 
 
@@ -1000,6 +1027,12 @@ static Instance make_instance()
     s.skinny = SKINNY;
     s.dmax = DMAX;
     for (int v = 0; v < kVariants; v++) s.fn[v] = nullptr;
+    s.guarded[0] = s.guarded[1] = nullptr;
+    // every operand fits nine digits, every int32 five: these instances can stand behind any speculative launch
+    if constexpr (NA == 9 && !SKINNY && DMAX == 16 && !B32ONLY && !BPLONLY) {
+        if constexpr (NB == 9) s.guarded[0] = gemm_mfma_guarded_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, DMAX>;
+        if constexpr (NB == 5) s.guarded[1] = gemm_mfma_guarded_kernel<NA, NB, WVM, WVN, WM, WN, KK, true, DMAX>;
+    }
     if constexpr (BPLONLY) {
         static_assert(SKINNY && !B32ONLY, "grouped launches run on the 32-row tiles");
         s.fn[kB64GroupBPlanes] = gemm_mfma_kernel<NA, NB, WVM, WVN, WM, WN, KK, false, false, false, true, false, DMAX, true>;
