@@ -36,7 +36,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20, help="untimed calls before the timed steps (at least; see SPIN_UP_MS)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,small,cpu,calib (default gemm,extra,cpu; small = configs 1 and 2 of extra alone)")
+    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,small,cold,cpu,calib (default gemm,extra,cpu; small = configs 1 and 2 of extra alone, cold = the calls on operands never seen alone)")
     return ap.parse_args()
 
 
@@ -277,40 +277,7 @@ def run():
         extra[nm] = gemm_leg(K, H2, W22, 16, 100, 10, samples, nm, host=(H2_h, W22_h))
         del X2, W21, H2, W22, X2_h, W21_h, H2_h, W22_h
 
-    if "extra" in legs:
-        # config 4, full-range operands (two's-complement wraparound)
-        g4 = torch.Generator(device="cpu").manual_seed(4001)
-        Af_h = full_range(g4, (1, M, Kd))
-        Wf_h = full_range(g4, (N, Kd))
-        Af, Wf = Af_h.cuda(), Wf_h.cuda()
-        nm = "gemm_config4_full_range"
-        extra[nm] = gemm_leg(K, Af, Wf, 29, max(3, args.steps // 4), 1, samples, nm)
-        # the same product modulo 2^64 (shift 0): only the digit pairs below 2^64 are multiplied; torch's CPU matmul wraps
-        # the same way, so this variant is checked against the reference's CPU path itself
-        nm = "gemm_config4_full_range_shift0"
-        extra[nm] = gemm_leg(K, Af, Wf, 0, max(3, args.steps // 4), 1, samples, nm, host=(Af_h, Wf_h))
-        full_range_host = (Af_h, Wf_h[:256].clone())        # the CPU leg times the reference's path on these too
-        del Af, Wf, Af_h, Wf_h
-        # real-model operand widths: Q31 activations (|x| < 2^37), int32 weights
-        Am = randint(g4, -(1 << 37), 1 << 37, (1, M, Kd)).cuda()
-        Wm = randint(g4, -(1 << 31), 1 << 31, (N, Kd)).to(torch.int32).cuda()
-        nm = "gemm_config4_q31_x_int32"
-        extra[nm] = gemm_leg(K, Am, Wm, 30, max(3, args.steps // 2), 1, samples, nm)
-        del Am, Wm
-        # the headline shape with the weights prepared once as digit planes (zk_gemm_prepare_weights): what a model
-        # with static weights gets; the one-time preparation is timed separately and is NOT part of `value`
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        K.prepare_weights(W[0] if W.dim() == 3 else W)
-        prep_ms = (time.perf_counter() - t0) * 1e3
-        extra["gemm_config4_prepared_weights"] = gemm_leg(K, A, W, c, args.steps, 5, samples, "gemm_config4_prepared_weights", host=(A_h, W_h))
-        extra["gemm_config4_prepared_weights"]["prepare_once_ms"] = prep_ms
-        K.release_weights(W[0] if W.dim() == 3 else W)
-        # other instruction path on the headline shape, for the comparison
-        K.lib.zk_gemm_set_path(1 if path == 2 else 2)
-        extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1, samples, "gemm_config4_other_path", host=(A_h, W_h))
-        K.lib.zk_gemm_set_path(0)
-
+    if legs & {"extra", "cold"}:
         # Calls on operands the library has not seen.  The reference's driver builds every layer anew on the device for
         # every position (inference/generate.py:227-238) and loads each routed expert from disk when it is hit
         # (inference/model.py:1362-1363), so in an unchanged drop-in the weight pointers of most calls are new, or are
@@ -373,6 +340,40 @@ def run():
         cold_leg("cold_gemm_config2_w1_128x7168x2048", 128, 7168, 2048, 16)
         cold_leg("cold_gemm_config1_16x7168x576", 16, 7168, 576, 29)
         torch.cuda.empty_cache()
+
+    if "extra" in legs:
+        # config 4, full-range operands (two's-complement wraparound)
+        g4 = torch.Generator(device="cpu").manual_seed(4001)
+        Af_h = full_range(g4, (1, M, Kd))
+        Wf_h = full_range(g4, (N, Kd))
+        Af, Wf = Af_h.cuda(), Wf_h.cuda()
+        nm = "gemm_config4_full_range"
+        extra[nm] = gemm_leg(K, Af, Wf, 29, max(3, args.steps // 4), 1, samples, nm)
+        # the same product modulo 2^64 (shift 0): only the digit pairs below 2^64 are multiplied; torch's CPU matmul wraps
+        # the same way, so this variant is checked against the reference's CPU path itself
+        nm = "gemm_config4_full_range_shift0"
+        extra[nm] = gemm_leg(K, Af, Wf, 0, max(3, args.steps // 4), 1, samples, nm, host=(Af_h, Wf_h))
+        full_range_host = (Af_h, Wf_h[:256].clone())        # the CPU leg times the reference's path on these too
+        del Af, Wf, Af_h, Wf_h
+        # real-model operand widths: Q31 activations (|x| < 2^37), int32 weights
+        Am = randint(g4, -(1 << 37), 1 << 37, (1, M, Kd)).cuda()
+        Wm = randint(g4, -(1 << 31), 1 << 31, (N, Kd)).to(torch.int32).cuda()
+        nm = "gemm_config4_q31_x_int32"
+        extra[nm] = gemm_leg(K, Am, Wm, 30, max(3, args.steps // 2), 1, samples, nm)
+        del Am, Wm
+        # the headline shape with the weights prepared once as digit planes (zk_gemm_prepare_weights): what a model
+        # with static weights gets; the one-time preparation is timed separately and is NOT part of `value`
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        K.prepare_weights(W[0] if W.dim() == 3 else W)
+        prep_ms = (time.perf_counter() - t0) * 1e3
+        extra["gemm_config4_prepared_weights"] = gemm_leg(K, A, W, c, args.steps, 5, samples, "gemm_config4_prepared_weights", host=(A_h, W_h))
+        extra["gemm_config4_prepared_weights"]["prepare_once_ms"] = prep_ms
+        K.release_weights(W[0] if W.dim() == 3 else W)
+        # other instruction path on the headline shape, for the comparison
+        K.lib.zk_gemm_set_path(1 if path == 2 else 2)
+        extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1, samples, "gemm_config4_other_path", host=(A_h, W_h))
+        K.lib.zk_gemm_set_path(0)
 
         # memory-bound kernels, 16 algorithmic bytes per element
         K.softmax_init_q19()

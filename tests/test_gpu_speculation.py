@@ -177,7 +177,9 @@ def test_stale_guess_both_kinds_of_guarded_launch(K, oracle, fallback, w32, monk
                 W.h[...] = rand_i32(rng, W.h.shape, 31) if w32 else rand_i64(rng, W.h.shape, 63)
                 A.d.copy_(torch.from_numpy(A.h))
                 W.d.copy_(torch.from_numpy(W.h))
-            pokes = [widen, lambda: A.poke((Bd - 1, M - 1, Kd - 1), -(1 << 62)), lambda: W.poke((N - 1, 0), (1 << 30) if w32 else (1 << 62))]
+            # (values of up to five digits make the guarded launch multiply with (5,5), wider ones with nine digits)
+            pokes = [widen, lambda: A.poke((Bd - 1, M - 1, Kd - 1), -(1 << 62)), lambda: W.poke((N - 1, 0), (1 << 30) if w32 else (1 << 62)),
+                     lambda: A.poke((0, 0, 1), 1 << 37), lambda: W.poke((1, Kd - 1), -(1 << 29) if w32 else -(1 << 36))]
             _stale_guess_rounds(K, _bmm(K, A, W, c), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 1, c), [A, W], pokes)
         # without a remainder
         A = Operand(rand_i64(rng, (1, 70, 200), 20))

@@ -335,7 +335,8 @@ __global__ __launch_bounds__(256) void a_planes_kernel(MfmaParams p, unsigned ch
 }
 
 // Folds the per-workgroup ranges of the plane pre-pass (`mm`, A only) and of the GEMM kernel (`wg`, A and B) into
-// range[0..3] and leaves the verdict in range[4]: 0 when `na` and `nb` digits covered them, 1 otherwise.
+// range[0..3] and leaves the verdict in range[4]: 0 when `na` and `nb` digits covered them, otherwise 1 when five digits
+// cover both operands and 2 when they do not (what the guarded launch behind the product multiplies with).
 // `host_copy`, when set, is pinned host memory that receives the same five words.
 // `parts` workgroups (of any size) share the slots; each leaves its partial result in `scratch` and takes a ticket, and
 // the one that arrives last folds the partials (a launch with tens of thousands of tiles would otherwise spend longer
@@ -405,7 +406,7 @@ __device__ __forceinline__ void range_fold_body(const FoldArgs &f, int part)
     for (int q = 0; q < 4; q++) f.range[q] = v[q];
     const int need_a = limbs_needed((int64_t)(v[0] ^ kSignFlip), (int64_t)(v[1] ^ kSignFlip));
     const int need_b = limbs_needed((int64_t)(v[2] ^ kSignFlip), (int64_t)(v[3] ^ kSignFlip));
-    const unsigned long long verdict = (need_a <= f.na && need_b <= f.nb) ? 0ull : 1ull;
+    const unsigned long long verdict = (need_a <= f.na && need_b <= f.nb) ? 0ull : ((need_a <= 5 && need_b <= 5) ? 1ull : 2ull);
     f.range[4] = verdict;
     if (f.host_copy) {
 #pragma unroll
@@ -921,7 +922,17 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_kernel(MfmaParams p)
 template <int NA, int NB, int WVM, int WVN, int WM, int WN, int KK, bool B32, int DMAX = 16>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm_mfma_guarded_kernel(MfmaParams p)
 {
-    if (__atomic_load_n(p.guard, __ATOMIC_RELAXED) == 0) return;            // (the same for every thread of the launch)
+    const unsigned long long verdict = __atomic_load_n(p.guard, __ATOMIC_RELAXED);            // (the same for every thread of the launch)
+    if (verdict == 0) return;
+    if (verdict == 1 && (NA > 5 || NB > 5)) {
+        // five digits cover both operands (the fold kernel has seen every element): a third of the digit pairs of (9,9)
+        constexpr int NA5 = NA > 5 ? 5 : NA, NB5 = NB > 5 ? 5 : NB;
+        for (int block = (int)blockIdx.x; block < p.walk_blocks; block += (int)gridDim.x) {
+            gemm_mfma_block<NA5, NB5, WVM, WVN, WM, WN, KK, B32, false, false, false, false, 16, false>(p, block);
+            __syncthreads();
+        }
+        return;
+    }
     for (int block = (int)blockIdx.x; block < p.walk_blocks; block += (int)gridDim.x) {
         gemm_mfma_block<NA, NB, WVM, WVN, WM, WN, KK, B32, false, false, false, false, DMAX, false>(p, block);
         __syncthreads();            // (the LDS stages and the range words in them are used again)
