@@ -149,7 +149,7 @@ static RangeCache g_cache;
 // behind a speculative one is always the vector-ALU kernel; ZK_B_ROWS_MIN_MACS: product
 // size from which a small n-contiguous int64 B is rewritten with contiguous rows first; ZK_SKINNY_MAX_M: rows up to
 // which the 32-row tiles are used.
-struct Switches { bool sync_verdict, no_tail_split, valu_fallback; double b_rows_min_macs; int skinny_max_m; };
+struct Switches { bool sync_verdict, no_tail_split, valu_fallback; double b_rows_min_macs; int skinny_max_m, planes_min_tiles_n; };
 constexpr long kBRowsMinMacs = 1L << 32;
 constexpr double kShapeGuessMaxMacs = 17179869184.0;        // 2^34: about 0.15 ms on the matrix pipe
 // Rows up to which a product runs on the 32-row tiles (two of them from 33 rows on): measured against the 128-row tiles,
@@ -165,6 +165,8 @@ static Switches read_switches()
     s.b_rows_min_macs = m ? atof(m) : (double)kBRowsMinMacs;
     const char *sk = getenv("ZK_SKINNY_MAX_M");
     s.skinny_max_m = sk ? atoi(sk) : kSkinnyMaxRows;
+    const char *pt = getenv("ZK_PLANES_MIN_TILES_N");
+    s.planes_min_tiles_n = pt ? atoi(pt) : 4;
     return s;
 }
 static Switches g_switches = read_switches();
@@ -653,7 +655,9 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         if (total > 0x7FFFFFFFL / 8) return kDeclined;
         // A is pre-split into digit planes when enough column tiles reuse it to pay for the extra pass (never for the
         // 32-row tiles: splitting a handful of rows on the fly is cheaper than another kernel in front)
-        const bool use_planes = !kmajor && (p.tiles_n >= 4 || prep) && !inst->skinny;
+        // (nor for a launch with fewer tiles than compute units: its tiles are cut along K, every workgroup splits a short
+        // slice of A, and the pre-pass would be a launch of its own in front: 128 rows x [2048,7168] 43.8 -> 42.4 us)
+        const bool use_planes = !kmajor && ((p.tiles_n >= g_switches.planes_min_tiles_n && total >= g_cache.cus) || prep) && !inst->skinny;
         if (b_shift && (kmajor || !inst->skinny)) return kDeclined;
         const int variant = prep ? (inst->skinny ? kB64FlyBPlanes : kB64PlanesBoth)
                           : b_shift ? (d.b32 ? kB32FlyRs : kB64FlyRs)
