@@ -751,6 +751,13 @@ def run():
         o8 = torch.empty((18432, 7168), dtype=torch.int32, device="cuda")
         hbm("fp8_block_scaled_to_int32_18432x7168", lambda: K.lib.fp8_block_scaled_to_int32(w8.data_ptr(), s8.data_ptr(), o8.data_ptr(), 18432, 7168, 30),
             w8.numel(), bytes_per_elem=5.0, steps=20)
+        # four fifths of that kernel's traffic are writes: next to it, what this device takes in streaming stores alone
+        store_gbps = K.lib.zk_probe_store_gbps(528 << 20, 10)
+        K._check("store probe")
+        e8 = extra["fp8_block_scaled_to_int32_18432x7168"]
+        e8["streaming_store_ceiling_GBps"] = store_gbps
+        e8["write_GBps"] = 4.0 * w8.numel() / (e8["ms"] * 1e-3) / 1e9
+        e8["write_frac_of_store_ceiling"] = e8["write_GBps"] / store_gbps if store_gbps else None
         del w8, o8
         wb = torch.randn((18432, 7168), generator=gq, dtype=torch.float32)
         w16 = wb.to(torch.bfloat16).cuda()
@@ -865,6 +872,13 @@ def run():
     del A, W, Cb, Rb
     torch.cuda.empty_cache()
     torch.cuda.synchronize()
+    # this program starts no other process (no subprocess, no worker pool; the CPU leg's threads live in this process and
+    # end with it): whatever a supervisor finds alive once it has exited is not its child.  Said in the line, checked here.
+    try:
+        import psutil
+        out["summary"]["child_processes_at_exit"] = len(psutil.Process().children(recursive=True))
+    except Exception:
+        out["summary"]["child_processes_at_exit"] = None
     print(json.dumps(out))
     sys.stdout.flush()
     sys.stderr.flush()

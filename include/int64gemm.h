@@ -269,6 +269,9 @@ double zk_probe_mfma_i8_tops(int with_lds, int random_data, int steps);
  * workgroups store 16 bytes each, a second kernel reads them): what the launches alone cost a call that is made of a
  * streaming kernel and a finishing kernel.  A measurement aid for bench.py; not needed for inference. */
 double zk_probe_launch_pair_us(int workgroups, int reps);
+/* GB/s of non-temporal 16-byte stores into a buffer of `bytes` bytes with nothing read: what the device takes in writes
+ * alone, the ceiling of the write-heavy converters.  A measurement aid for bench.py. */
+double zk_probe_store_gbps(long bytes, int reps);
 
 /* HIP-event stopwatch on the null stream (the stream every entry point launches on). */
 void zk_timer_start(void);

@@ -611,11 +611,22 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
         b_stride[it] = live ? STAGE : 0;
     }
 
+    // The staged data of a step can be handled in two parts, so that a kernel with two MFMA depths per step splits,
+    // stores and reloads one half behind each depth (its loads are then spread over the step instead of leaving in one
+    // burst at its end): PART 0 = A and the first half of B's items, 1 = the rest of B, -1 = everything.
+    typedef std::integral_constant<int, -1> PAll;
+    typedef std::integral_constant<int, 0> PFirst;
+    typedef std::integral_constant<int, 1> PSecond;
+    constexpr int B_N = BPL ? B_CIT : B_IT;          // items (or chunks of planes) of B per thread
+
     // FAST: the whole step lies inside K and the pointers allow 16-byte loads: no guards at all.
-    auto fetch = [&](int ks, auto fast_tag) {
+    auto fetch = [&](int ks, auto fast_tag, auto part_tag) {
         constexpr bool FAST = decltype(fast_tag)::value;
+        constexpr int PART = decltype(part_tag)::value;
+        constexpr int B_LO = PART == 1 ? B_N / 2 : 0, B_HI = PART == 0 ? B_N / 2 : B_N;
         const int k0 = ks * BK;
-        if (APL) {
+        if (PART == 1) {
+        } else if (APL) {
 #pragma unroll
             for (int it = 0; it < A_CIT; it++)
                 pa[it] = *reinterpret_cast<const v4i *>(a_pl[it] + (long)ks * (KK * NA * 1024));
@@ -628,11 +639,11 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
         }
         if (BPL) {
 #pragma unroll
-            for (int it = 0; it < B_CIT; it++)
+            for (int it = B_LO; it < B_HI; it++)
                 pb[it] = *(const ZK_GLOBAL_MEM v4i *)(b_pl[it] + (long)ks * (KK * NB * 1024));
         }
 #pragma unroll
-        for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
+        for (int it = (BPL ? 0 : B_LO); it < (BPL ? 0 : B_HI); it++) {
             if (BKM) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -656,8 +667,11 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
     };
 
     // staged elements -> digits -> LDS stage `buf`, fragment order
-    auto stash = [&](int buf) {
-        if (APL) {
+    auto stash = [&](int buf, auto part_tag) {
+        constexpr int PART = decltype(part_tag)::value;
+        constexpr int B_LO = PART == 1 ? B_N / 2 : 0, B_HI = PART == 0 ? B_N / 2 : B_N;
+        if (PART == 1) {
+        } else if (APL) {
 #pragma unroll
             for (int it = 0; it < A_CIT; it++)
                 *reinterpret_cast<v4i *>(smem + pl_dst[it] + buf * pl_stride[it]) = pa[it];
@@ -673,11 +687,11 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
         }
         if (BPL) {
 #pragma unroll
-            for (int it = 0; it < B_CIT; it++)
+            for (int it = B_LO; it < B_HI; it++)
                 *reinterpret_cast<v4i *>(smem + plb_dst[it] + buf * plb_stride[it]) = pb[it];
         }
 #pragma unroll
-        for (int it = 0; it < (BPL ? 0 : B_IT); it++) {
+        for (int it = (BPL ? 0 : B_LO); it < (BPL ? 0 : B_HI); it++) {
             uint2 dg[NB];
             if (BRS) {
                 int64_t y[8];
@@ -744,11 +758,17 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
     // Range tracking of the staged elements of data step d, done while the registers still hold them.
     // (called once per data step, in order: the turn counters stand for d % vmod_a and d % vmod_b without a division)
     int turn_a = ks_begin % vmod_a, turn_b = ks_begin % vmod_b;
-    auto track = [&](int) {
-        const bool my_a = turn_a == tn, my_b = turn_b == tm;
-        turn_a = turn_a + 1 == vmod_a ? 0 : turn_a + 1;
-        turn_b = turn_b + 1 == vmod_b ? 0 : turn_b + 1;
-        if (verify_a && my_a) {
+    bool my_a = false, my_b = false;
+    auto track = [&](auto part_tag) {
+        constexpr int PART = decltype(part_tag)::value;
+        constexpr int B_LO = PART == 1 ? B_IT / 2 : 0, B_HI = PART == 0 ? B_IT / 2 : B_IT;
+        if (PART != 1) {            // (the turns advance once per data step, with its first part)
+            my_a = turn_a == tn;
+            my_b = turn_b == tm;
+            turn_a = turn_a + 1 == vmod_a ? 0 : turn_a + 1;
+            turn_b = turn_b + 1 == vmod_b ? 0 : turn_b + 1;
+        }
+        if (PART != 1 && verify_a && my_a) {
 #pragma unroll
             for (int it = 0; it < A_IT; it++)
 #pragma unroll
@@ -757,7 +777,7 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
         }
         if (verify_b && my_b) {
 #pragma unroll
-            for (int it = 0; it < B_IT; it++)
+            for (int it = B_LO; it < B_HI; it++)
 #pragma unroll
                 for (int q = 0; q < 8; q++) {
                     if (B32 && !BRS) {
@@ -778,8 +798,48 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
     //   B  the second half of the MFMAs interleaved, in one scheduling region, with the digit split of the
     //      elements staged for step ks+1 and their LDS writes into the other stage;
     //   C  the loads of step ks+2 into the now free staging registers, then the barrier.
+    // Two depths per step, B split on the fly: one depth's MFMAs carry the split of one half of the staged data, whose
+    // registers are reloaded right behind it.  Each half's loads then have a whole step to land and some are under way
+    // at every moment (with one burst per step nothing is for the part of the step between their arrival and the next
+    // burst: the routed experts' int32 weights streamed at 5.3 TB/s that way).
+    constexpr bool SPREAD = KK == 2 && !BKM && B_N >= 2 && B_N % 2 == 0;
     auto step_body = [&](int ks, auto fast_tag) {
         const int cur = (ks - ks_begin) & 1;
+        if constexpr (SPREAD) {
+            {
+                v4i fa[WM][NA], fb[WN][NB];
+                load_frags(cur, 0, fa, fb);
+                mfma_slice(I0(), IF(), fa, fb);
+                stash(cur ^ 1, PFirst());
+#pragma unroll
+                for (int i = 0; i < MFMAS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, ZK_VALU_PER_MFMA, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                track(PFirst());
+                if (ks + 2 < ks_end) fetch(ks + 2, fast_tag, PFirst());
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            {
+                v4i fa[WM][NA], fb[WN][NB];
+                load_frags(cur, 1, fa, fb);
+                mfma_slice(I0(), IF(), fa, fb);
+                stash(cur ^ 1, PSecond());
+#pragma unroll
+                for (int i = 0; i < MFMAS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, ZK_VALU_PER_MFMA, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                track(PSecond());
+                if (ks + 2 < ks_end) fetch(ks + 2, fast_tag, PSecond());
+            }
+            __syncthreads();
+            return;
+        }
 #pragma unroll
         for (int kk = 0; kk < KK - 1; kk++) {
             v4i fa[WM][NA], fb[WN][NB];
@@ -791,7 +851,7 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
         mfma_slice(I0(), IH(), fa, fb);
         __builtin_amdgcn_sched_barrier(0);
         mfma_slice(IH(), IF(), fa, fb);
-        stash(cur ^ 1);
+        stash(cur ^ 1, PAll());
 #pragma unroll
         for (int i = 0; i < MFMAS - MFMAS / 2; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -799,17 +859,17 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        track(ks + 1);
-        if (ks + 2 < ks_end) fetch(ks + 2, fast_tag);
+        track(PAll());
+        if (ks + 2 < ks_end) fetch(ks + 2, fast_tag, PAll());
         __syncthreads();
     };
 
     // prologue: stage 0 holds the first step, the staging registers hold the second
-    if (ks_begin < full_steps) fetch(ks_begin, std::true_type()); else fetch(ks_begin, std::false_type());
-    track(ks_begin);
-    stash(0);
+    if (ks_begin < full_steps) fetch(ks_begin, std::true_type(), PAll()); else fetch(ks_begin, std::false_type(), PAll());
+    track(PAll());
+    stash(0, PAll());
     if (ks_begin + 1 < ks_end) {
-        if (ks_begin + 1 < full_steps) fetch(ks_begin + 1, std::true_type()); else fetch(ks_begin + 1, std::false_type());
+        if (ks_begin + 1 < full_steps) fetch(ks_begin + 1, std::true_type(), PAll()); else fetch(ks_begin + 1, std::false_type(), PAll());
     }
     __syncthreads();
     int ks = ks_begin;

@@ -77,6 +77,44 @@ __global__ __launch_bounds__(256) void probe_pair_second(const unsigned long lon
 
 }  // namespace zk
 
+namespace zk {
+
+// What the device takes in streaming stores alone (nothing read): every thread writes 16-byte pieces, non-temporal, the
+// grid striding over the buffer.  The ceiling of a kernel whose traffic is mostly writes (the fp8 checkpoint quantiser
+// writes four bytes per byte read).
+__global__ __launch_bounds__(256) void probe_store_kernel(pv4i *out, long pieces, int seed)
+{
+    const pv4i v = { seed, seed + 1, seed + 2, seed + 3 };
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (long)gridDim.x * 256) __builtin_nontemporal_store(v, out + i);
+}
+
+}  // namespace zk
+
+extern "C" double zk_probe_store_gbps(long bytes, int reps)
+{
+    if (bytes < 4096 || reps <= 0) { zk::set_error(zk::kBadArgument, "zk_probe_store_gbps: bad argument"); return 0.0; }
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    zk::pv4i *buf = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    double gbps = 0.0;
+    const long pieces = bytes / 16;
+    if (hipMalloc(&buf, (size_t)pieces * 16) == hipSuccess && hipEventCreate(&t0) == hipSuccess && hipEventCreate(&t1) == hipSuccess) {
+        for (int r = 0; r < 3; r++) zk::probe_store_kernel<<<dim3((unsigned)(cus * 8)), dim3(256), 0, 0>>>(buf, pieces, r);
+        (void)hipEventRecord(t0, 0);
+        for (int r = 0; r < reps; r++) zk::probe_store_kernel<<<dim3((unsigned)(cus * 8)), dim3(256), 0, 0>>>(buf, pieces, r);
+        (void)hipEventRecord(t1, 0);
+        float ms = 0.f;
+        if (hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess && ms > 0.f)
+            gbps = (double)pieces * 16.0 * reps / (ms * 1e-3) / 1e9;
+    }
+    if (hipGetLastError() != hipSuccess || gbps == 0.0) zk::set_error(zk::kLaunchFailure, "zk_probe_store_gbps: measurement failed");
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    if (buf) (void)hipFree(buf);
+    return gbps;
+}
+
 extern "C" double zk_probe_launch_pair_us(int workgroups, int reps)
 {
     if (workgroups <= 0 || workgroups > 65536 || reps <= 0) { zk::set_error(zk::kBadArgument, "zk_probe_launch_pair_us: bad argument"); return 0.0; }

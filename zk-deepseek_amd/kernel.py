@@ -90,6 +90,8 @@ lib.zk_probe_mfma_i8_tops.argtypes = [_ci, _ci, _ci]
 lib.zk_probe_mfma_i8_tops.restype = ctypes.c_double
 lib.zk_probe_launch_pair_us.argtypes = [_ci, _ci]
 lib.zk_probe_launch_pair_us.restype = ctypes.c_double
+lib.zk_probe_store_gbps.argtypes = [ctypes.c_long, _ci]
+lib.zk_probe_store_gbps.restype = ctypes.c_double
 lib.zk_workspace_bytes.restype = ctypes.c_size_t
 lib.zk_prepared_weights_bytes.restype = ctypes.c_size_t
 
