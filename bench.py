@@ -7,8 +7,9 @@ Prints ONE JSON line.  `value` is the int64 GEMM throughput (Gmac/s) of benchmar
 (512 x 7168 against W[18432,7168], config-1 operand ranges, shift 29) through the C ABI with operands
 resident in HBM; one step = one call of int64_64_bmm_broadcast_launcher.  The same line carries the
 other shapes the metric names (config-1 GEMM, full-range config 4, softmax / SiLU / sigmoid / RMSNorm
-HBM GB/s) under "extra", the roofline of the dominant kernel (and, under "roofline_others", of the HBM-bound
-shapes the metric names), and a CPU baseline timed on this host.
+HBM GB/s) under "extra", the roofline of the dominant kernel (with the figures of config 1 and of the HBM-bound
+shapes the metric names as flat keys inside it, and once more at the end of the line under "summary"), the calls on
+operands never seen (--only cold), and a CPU baseline timed on this host.
 
 Nothing is timed before it has been checked: the headline product is compared with torch's int64 matmul on the CPU
 (same input bytes) on a block of columns before the timed loop starts, and the run aborts on a mismatch; the other
