@@ -234,10 +234,11 @@ void zk_gemm_last_plan(int *path, int *limbs_a, int *limbs_b);
  * limbs_a * limbs_b; fewer when the stored bits [shift, shift + 64) of the sum lie below the weight of the top
  * digit pairs, which are then not multiplied at all. */
 int zk_gemm_last_pairs(void);
-/* The MFMA path guesses how many base-256 digits the operands need and checks the guess on the device.  A call
- * whose operands (pointer, shape) were seen before does not wait for that check: a guarded vector-ALU launch
- * behind it recomputes the outputs if the guess was too small.  This returns how many calls so far needed that
- * recomputation (counted once their ranges have reached the host; it waits for nothing). */
+/* The MFMA path guesses how many base-256 digits the operands need (from what the same pointers, or the last operands
+ * of the same shape, needed) and checks the guess on the device.  No call waits for that check: a guarded launch
+ * behind it (the widest MFMA instance, or the vector-ALU tiles where that does not apply) recomputes the outputs if the
+ * guess was too small.  This returns how many calls so far needed that recomputation (counted once their ranges have
+ * reached the host; it waits for nothing). */
 long zk_gemm_guard_hits(void);
 /* How many int64_grouped_bmm_launcher calls so far ran as ONE launch over all groups (the others went group by group). */
 long zk_gemm_grouped_mfma_calls(void);
