@@ -385,6 +385,12 @@ def run():
             K._check(name)
             gbs = (nelem * bytes_per_elem + extra_bytes) / (ms * 1e-3) / 1e9
             extra[name] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS, "elements": nelem}
+            if ms < 0.05 and launch_floor_us:
+                # a launch this short is bound by the launch itself as much as by its bytes: next to the HBM fraction,
+                # the fraction of (one launch as measured on this device + the bytes at the HBM peak)
+                floor_us = launch_floor_us / 2.0 + (nelem * bytes_per_elem + extra_bytes) / (HBM_PEAK_GBS * 1e9) * 1e6
+                extra[name]["one_launch_us"] = launch_floor_us / 2.0
+                extra[name]["frac_of_launch_plus_hbm_floor"] = floor_us / (ms * 1e3)
             if sample is not None:
                 samples.append((name, sample()))
 
@@ -824,6 +830,12 @@ def run():
                           "traffic": None, "note": "16 algorithmic bytes per element (8 read + 8 written)"}
             flat[nm + "_GBps"] = e["GBps"]
             flat[nm + "_frac_hbm"] = e["frac_hbm_peak"]
+            if "frac_of_launch_plus_hbm_floor" in e:
+                flat[nm + "_frac_of_launch_plus_hbm_floor"] = e["frac_of_launch_plus_hbm_floor"]
+    for nm in ("gemm_1token_wkv_a_7168x576_int32",):
+        if nm in extra and "frac_of_launch_plus_hbm_floor" in extra[nm]:
+            flat[nm + "_us"] = extra[nm]["ms"] * 1e3
+            flat[nm + "_frac_of_launch_plus_hbm_floor"] = extra[nm]["frac_of_launch_plus_hbm_floor"]
     for nm in ("moe_experts_int32_256tok_top8_of_256", "moe_experts_config5_256tok_top8_of_256"):
         if nm in extra:
             flat[nm + "_frac_hbm"] = extra[nm]["frac_hbm_peak"]
