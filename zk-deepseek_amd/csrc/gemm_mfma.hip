@@ -33,6 +33,10 @@
 
 namespace zk {
 
+// the streamed form of the grouped launch for int32 weights (gemm_stream32.h), by digit counts; null: none
+MfmaKernel stream32_grouped_kernel(int na, int nb, size_t *lds);
+MfmaKernel stream32_grouped_kernel_wide(int na, int nb, size_t *lds);
+
 // Digit-count combinations that are compiled.  A request is rounded up to the cheapest one that covers it.
 static const Instance *instances(int *count)
 {
@@ -146,10 +150,11 @@ static RangeCache g_cache;
 
 // Diagnosis switches, read from the environment once when the library is loaded (and again on zk_reload_env):
 // ZK_GEMM_SYNC: every call waits for its own digit verdict; ZK_NO_TAIL_SPLIT: no split-K; ZK_VALU_FALLBACK: the guarded launch
-// behind a speculative one is always the vector-ALU kernel; ZK_B_ROWS_MIN_MACS: product
+// behind a speculative one is always the vector-ALU kernel; ZK_NO_STREAM32: grouped launches on int32 weights keep the general
+// 32-row kernel; ZK_B_ROWS_MIN_MACS: product
 // size from which a small n-contiguous int64 B is rewritten with contiguous rows first; ZK_SKINNY_MAX_M: rows up to
 // which the 32-row tiles are used.
-struct Switches { bool sync_verdict, no_tail_split, valu_fallback; double b_rows_min_macs; int skinny_max_m, planes_min_tiles_n; };
+struct Switches { bool sync_verdict, no_tail_split, valu_fallback, no_stream32; double b_rows_min_macs; int skinny_max_m, planes_min_tiles_n, stream32_min_pairs; };
 constexpr long kBRowsMinMacs = 1L << 32;
 constexpr double kShapeGuessMaxMacs = 17179869184.0;        // 2^34: about 0.15 ms on the matrix pipe
 // Rows up to which a product runs on the 32-row tiles (two of them from 33 rows on): measured against the 128-row tiles,
@@ -161,6 +166,9 @@ static Switches read_switches()
     s.sync_verdict = getenv("ZK_GEMM_SYNC") != nullptr;
     s.no_tail_split = getenv("ZK_NO_TAIL_SPLIT") != nullptr;
     s.valu_fallback = getenv("ZK_VALU_FALLBACK") != nullptr;
+    s.no_stream32 = getenv("ZK_NO_STREAM32") != nullptr;
+    const char *sp = getenv("ZK_STREAM32_MIN_PAIRS");
+    s.stream32_min_pairs = sp ? atoi(sp) : 16;
     const char *m = getenv("ZK_B_ROWS_MIN_MACS");
     s.b_rows_min_macs = m ? atof(m) : (double)kBRowsMinMacs;
     const char *sk = getenv("ZK_SKINNY_MAX_M");
@@ -866,6 +874,17 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         if (!inst) return 1;
         MfmaKernel fn = inst->fn[prep ? kB64GroupBPlanes : (d.b32 ? kB32Group : kB64Group)];
         if (!fn) return 1;
+        // int32 weights, whole steps, rows of A on 16-byte boundaries, sixteen digit pairs or more: the form that streams the
+        // weights through LDS rings.  (Measured on 256 experts, one box, streamed against general: (3,4) digits 5.64
+        // against 5.86 TB/s at K = 7168 and level at K = 2048; (4,4) level at K = 7168 and 5.08 against 3.15 at K = 2048;
+        // (5,5) 4.18 against 3.87.  ZK_STREAM32_MIN_PAIRS moves the limit.)
+        size_t stream_lds = 0;
+        if (d.b32 && !prep && !g_switches.no_stream32 && d.K % 32 == 0 && (((uintptr_t)d.A | (uintptr_t)(d.lda * 8)) & 15) == 0 && inst->bn == 256 &&
+            inst->na * inst->nb >= g_switches.stream32_min_pairs) {
+            MfmaKernel sfn = stream32_grouped_kernel(inst->na, inst->nb, &stream_lds);
+            if (!sfn) sfn = stream32_grouped_kernel_wide(inst->na, inst->nb, &stream_lds);
+            if (sfn) fn = sfn; else stream_lds = 0;
+        }
         const long pairs = inst->na < inst->nb ? inst->na : inst->nb;
         const int ksteps = (d.K + 31) / 32;
         if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return 1;
@@ -876,7 +895,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         p.main_tiles = (int)blocks;
         if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;
         p.wg_range = g_cache.wg;
-        const size_t lds = 2 * (size_t)inst->kk * ((inst->bm / 32) * inst->na + (inst->bn / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
+        const size_t lds = stream_lds ? stream_lds : 2 * (size_t)inst->kk * ((inst->bm / 32) * inst->na + (inst->bn / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
         static std::set<const void *> lds_raised;
         if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
             if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {

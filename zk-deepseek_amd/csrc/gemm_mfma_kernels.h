@@ -550,6 +550,7 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
     // LDS destinations are stage-relative; threads with no work in an iteration aim at a dummy area behind the two
     // stages (and a zero stage stride), which keeps the loop body free of branches.
     constexpr int DUMMY = 2 * STAGE;
+    bool a_pad[A_IT];
     int a_j[A_IT], b_j[B_IT], a_dst[A_IT], b_dst[B_IT], pl_dst[A_CIT], plb_dst[B_CIT];
     int a_stride[A_IT], b_stride[B_IT], pl_stride[A_CIT], plb_stride[B_CIT];
     if (APL) {
@@ -573,6 +574,10 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
             const int row = (live ? idx : 0) / OCTS;
             a_j[it] = idx % OCTS;
             int m = m0 + row;
+            // (rows past the end are loaded from the last row, a valid address, and multiplied as zeros: the device is
+            // power managed and what the matrix pipe draws depends on the bits it is fed; an expert's tile has some
+            // 8 real rows of 32)
+            a_pad[it] = m >= m_lim;
             m = m < m_lim ? m : m_lim - 1;
             a_src[it] = p.A + (long)g * p.sA + (long)m * p.lda;
             a_dst[it] = live ? frag_offset(row, a_j[it], NA, SUBSTAGE) : DUMMY;
@@ -682,7 +687,7 @@ __device__ __forceinline__ void gemm_mfma_block(const MfmaParams &p, const int b
                 limb_split8<NA>(sa[it], dg);
 #pragma unroll
                 for (int i = 0; i < NA; i++)
-                    *reinterpret_cast<uint2 *>(smem + a_dst[it] + buf * a_stride[it] + i * 1024) = dg[i];
+                    *reinterpret_cast<uint2 *>(smem + a_dst[it] + buf * a_stride[it] + i * 1024) = a_pad[it] ? make_uint2(0u, 0u) : dg[i];
             }
         }
         if (BPL) {
