@@ -1265,6 +1265,91 @@ def test_int64_grouped_bmm_few_rows(K, oracle, w32, T, Kr, Kd, N):
         assert K.lib.zk_gemm_grouped_mfma_calls() == before and K.gemm_last_plan()[0] == 1
 
 
+@pytest.mark.parametrize("min_pairs", [None, "0"])
+@pytest.mark.parametrize("bits,top,Kd", [((20, 16), False, 224), ((28, 28), False, 224), ((37, 30), False, 96), ((36, 31), True, 224),
+                                         ((30, 31), True, 32), ((28, 24), False, 64)])
+def test_int64_grouped_bmm_int32_weights_streamed(K, oracle, monkeypatch, min_pairs, bits, top, Kd):
+    """the grouped launch that streams int32 weights through LDS rings (whole steps of K, sixteen digit pairs or more,
+    or any count with ZK_STREAM32_MIN_PAIRS=0): every pair of digit counts it is built for, fewer steps of K than the
+    ring has stages, experts with no rows, with one row and with more than a tile's 32, a ragged last tile column, the
+    remainder output, weights that reach INT32_MAX (a fifth digit); the first call reads its verdict back, the second
+    runs ahead of it behind a guarded launch"""
+    if min_pairs is None:
+        monkeypatch.delenv("ZK_STREAM32_MIN_PAIRS", raising=False)
+    else:
+        monkeypatch.setenv("ZK_STREAM32_MIN_PAIRS", min_pairs)
+    K.lib.zk_reload_env()
+    try:
+        rng = np.random.default_rng(bits[0] * 64 + bits[1] + Kd)
+        T, E, Kr, N = 90, 12, 3, 300
+        idx = _routing(rng, T, E, Kr)
+        idx[:60, 0] = 2                                       # expert 2: 60 rows, two tiles
+        idx[:60, 1:] = np.stack([rng.permutation([0, 1, 3, 4, 5])[: Kr - 1] for _ in range(60)])
+        x = rand_i64(rng, (T, Kd), bits[0])
+        ws = [rand_i32(rng, (N, Kd), bits[1]) for _ in range(E)]
+        if top:
+            ws[2][7, 5] = np.iinfo(np.int32).max
+            ws[4][299, Kd - 1] = np.iinfo(np.int32).min
+        K.lib.zk_gemm_set_path(2)
+        d = K.moe_dispatch(dev(idx), E)
+        xs = K.moe_gather_rows(dev(x), d)
+        seg, tok, _ = oracle.moe_dispatch(idx, E)
+        wd = [dev(w) for w in ws]
+        table = K.pointer_table(wd)
+        for c in (0, 19, 19):
+            streamed = K.lib.zk_gemm_grouped_streamed_calls()
+            C, R = K.int64_grouped_bmm(xs, table, True, N, c, d, want_remainder=True)
+            Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
+            assert np.array_equal(host(C), Ce), "quotient"
+            assert np.array_equal(host(R), Re), "remainder"
+        # (the first calls may run on digit counts that other operands left behind at these addresses; the last does not)
+        la, lb = K.gemm_last_plan()[1:]
+        assert la <= 5 and lb <= 5
+        took = K.lib.zk_gemm_grouped_streamed_calls() - streamed
+        assert took == (1 if min_pairs == "0" or la * lb >= 16 else 0), (la, lb, took)
+    finally:
+        K.lib.zk_gemm_set_path(0)
+        monkeypatch.delenv("ZK_STREAM32_MIN_PAIRS", raising=False)
+        K.lib.zk_reload_env()
+
+
+def test_int64_grouped_bmm_int32_weights_streamed_odd_operands(K, oracle, monkeypatch):
+    """what the streamed kernel does not take goes another way with the same bits: a K that is no multiple of 32, and one
+    expert's matrix at an address that is not a multiple of 16 (the kernel's workgroups for that expert report the full
+    range and the product is computed again on other kernels)"""
+    monkeypatch.setenv("ZK_STREAM32_MIN_PAIRS", "0")
+    K.lib.zk_reload_env()
+    try:
+        rng = np.random.default_rng(4242)
+        T, E, Kr, N = 40, 6, 2, 260
+        idx = _routing(rng, T, E, Kr)
+        seg, tok, _ = oracle.moe_dispatch(idx, E)
+        K.lib.zk_gemm_set_path(0)
+        d = K.moe_dispatch(dev(idx), E)
+        for Kd, shifted in ((200, False), (128, True)):
+            x = rand_i64(rng, (T, Kd), 30)
+            ws = [rand_i32(rng, (N, Kd), 27) for _ in range(E)]
+            xs = K.moe_gather_rows(dev(x), d)
+            wd = [dev(w) for w in ws]
+            if shifted:
+                flat = torch.zeros(N * Kd + 1, dtype=torch.int32, device="cuda")
+                flat[1:] = wd[3].reshape(-1)
+                wd[3] = flat[1:].view(N, Kd)
+                assert wd[3].data_ptr() % 16 == 4
+            table = K.pointer_table(wd)
+            streamed = K.lib.zk_gemm_grouped_streamed_calls()
+            for c in (0, 17):
+                C, R = K.int64_grouped_bmm(xs, table, True, N, c, d, want_remainder=True)
+                Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
+                assert np.array_equal(host(C), Ce), ("quotient", Kd, shifted, c)
+                assert np.array_equal(host(R), Re), ("remainder", Kd, shifted, c)
+            if not shifted:
+                assert K.lib.zk_gemm_grouped_streamed_calls() == streamed, "K % 32 != 0 is the general kernel's"
+    finally:
+        monkeypatch.delenv("ZK_STREAM32_MIN_PAIRS", raising=False)
+        K.lib.zk_reload_env()
+
+
 @pytest.mark.parametrize("w32", [False, True])
 def test_moe_experts(K, oracle, w32):
     """routed experts end to end (dispatch, gather, grouped gate/up GEMMs, SiLU gate, grouped down GEMM, weighted

@@ -253,6 +253,7 @@ long zk_gemm_guard_hits(void) { return zk::gemm_mfma_guard_hits(); }
 int zk_gemm_last_pairs(void) { return zk::g_last_digits ? zk::gemm_mfma_last_pairs() : 0; }
 
 long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
+long zk_gemm_grouped_streamed_calls(void) { return zk::gemm_mfma_grouped_streamed_calls(); }
 
 int zk_gemm_last_prepared(void) { return zk::g_last_digits ? zk::gemm_mfma_last_prepared() : 0; }
 int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K) { return zk::gemm_mfma_prepare(B, b32, groups, N, K); }

@@ -227,8 +227,10 @@ static void drain_pending()
 }
 
 static int g_last_pairs = 0, g_last_prepared = 0;
+static long g_streamed_calls = 0;
 int gemm_mfma_last_pairs() { return g_last_pairs; }
 int gemm_mfma_last_prepared() { return g_last_prepared; }
+long gemm_mfma_grouped_streamed_calls() { return g_streamed_calls; }
 
 long gemm_mfma_guard_hits()
 {
@@ -905,6 +907,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
             lds_raised.insert((const void *)fn);
         }
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
+        if (stream_lds) g_streamed_calls++;
         g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
         g_last_prepared = prep ? 1 : 0;
         {

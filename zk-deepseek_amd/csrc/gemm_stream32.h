@@ -163,26 +163,12 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
         split16_w32<NB>(x, fb);
         // this wavefront's eighth of A for the next step
         if (s + 1 < ksteps) stash_a(araw, (s + 1) & 1);
-#ifndef ZK_S32_NO_MFMA
 #pragma unroll
         for (int i = 0; i < NA; i++)
 #pragma unroll
             for (int j = 0; j < NB; j++)
-#ifdef ZK_S32_ZERO_MFMA
-                acc[i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(v4i{ 0, 0, 0, fa[i][0] & 1 }, v4i{ 0, 0, 0, fb[j][0] & 1 }, acc[i + j], 0, 0, 0);
-#else
                 acc[i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i + j], 0, 0, 0);
-#endif
-#else
-#pragma unroll
-        for (int i = 0; i < NA; i++) acc[0][i] += fa[i][0] + fb[i % NB][1];
-#ifdef ZK_S32_SLEEP
-        __builtin_amdgcn_s_sleep(ZK_S32_SLEEP);            // (64 clocks per unit)
-#endif
-#endif
-#ifndef ZK_S32_NO_BARRIER
         __syncthreads();
-#endif
     }
 
     // every workgroup leaves its ranges in its own slot; the waves' ranges meet in LDS (the rings are free by now)
