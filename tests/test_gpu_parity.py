@@ -1266,25 +1266,28 @@ def test_int64_grouped_bmm_few_rows(K, oracle, w32, T, Kr, Kd, N):
 
 
 @pytest.mark.parametrize("min_pairs", [None, "0"])
+@pytest.mark.parametrize("T", [90, 24])
 @pytest.mark.parametrize("bits,top,Kd", [((20, 16), False, 224), ((28, 28), False, 224), ((37, 30), False, 96), ((36, 31), True, 224),
-                                         ((30, 31), True, 32), ((28, 24), False, 64)])
-def test_int64_grouped_bmm_int32_weights_streamed(K, oracle, monkeypatch, min_pairs, bits, top, Kd):
+                                         ((30, 31), True, 32), ((28, 24), False, 64), ((28, 28), False, 160)])
+def test_int64_grouped_bmm_int32_weights_streamed(K, oracle, monkeypatch, min_pairs, T, bits, top, Kd):
     """the grouped launch that streams int32 weights through LDS rings (whole steps of K, sixteen digit pairs or more,
     or any count with ZK_STREAM32_MIN_PAIRS=0): every pair of digit counts it is built for, fewer steps of K than the
-    ring has stages, experts with no rows, with one row and with more than a tile's 32, a ragged last tile column, the
-    remainder output, weights that reach INT32_MAX (a fifth digit); the first call reads its verdict back, the second
-    runs ahead of it behind a guarded launch"""
+    ring has stages, an odd and an even number of steps, experts with no rows, with a few rows (tiles of at most 16 rows
+    multiply on v_mfma_i32_16x16x64_i8, two steps at a time) and with more than a tile's 32, a ragged last tile column,
+    the remainder output, weights that reach INT32_MAX (a fifth digit); the first call reads its verdict back, the
+    later ones run ahead of it behind a guarded launch"""
     if min_pairs is None:
         monkeypatch.delenv("ZK_STREAM32_MIN_PAIRS", raising=False)
     else:
         monkeypatch.setenv("ZK_STREAM32_MIN_PAIRS", min_pairs)
     K.lib.zk_reload_env()
     try:
-        rng = np.random.default_rng(bits[0] * 64 + bits[1] + Kd)
-        T, E, Kr, N = 90, 12, 3, 300
+        rng = np.random.default_rng(bits[0] * 64 + bits[1] + Kd + T)
+        E, Kr, N = 12, 3, 300
         idx = _routing(rng, T, E, Kr)
-        idx[:60, 0] = 2                                       # expert 2: 60 rows, two tiles
-        idx[:60, 1:] = np.stack([rng.permutation([0, 1, 3, 4, 5])[: Kr - 1] for _ in range(60)])
+        many = 2 * T // 3
+        idx[:many, 0] = 2                                     # expert 2: 60 rows (two tiles), or 16 (the most the 16-row form takes)
+        idx[:many, 1:] = np.stack([rng.permutation([0, 1, 3, 4, 5])[: Kr - 1] for _ in range(many)])
         x = rand_i64(rng, (T, Kd), bits[0])
         ws = [rand_i32(rng, (N, Kd), bits[1]) for _ in range(E)]
         if top:

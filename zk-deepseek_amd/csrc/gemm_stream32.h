@@ -116,12 +116,6 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
         }
     };
 
-    v16i acc[D];
-#pragma unroll
-    for (int d = 0; d < D; d++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[d][r] = 0;
-
     // prologue: the digits of A for step 0 straight from memory, the first steps on their way
     {
         const v4i a0 = *(const ZK_GLOBAL_MEM v4i *)(a_src);
@@ -132,43 +126,177 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
         if (d < ksteps) issue(d);
     __syncthreads();
 
-    for (int s = 0; s < ksteps; s++) {
+    // what every step begins with: its stage has landed (the loads of later steps may still be under way)
+    auto landed = [&](int s) {
         const int behind = ksteps - 1 - s;
         if (behind >= 2) wait_vmcnt<2 * kS32Loads>();
         else if (behind == 1) wait_vmcnt<kS32Loads>();
         else wait_vmcnt<0>();
-        asm volatile("" ::: "memory");                     // (the reads below stay behind the wait)
-        const unsigned st = (unsigned)(s % STG);
-        v4i raw[4], araw, fa[NA];
+        asm volatile("" ::: "memory");                     // (the reads that follow stay behind the wait)
+    };
+    auto track_b = [&](const v4i &v) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) raw[j] = *reinterpret_cast<const v4i *>(ring_b + st * 4096 + b_rd[j]);
-        araw = *reinterpret_cast<const v4i *>(ring_a + st * 8192 + wave * 1024 + lane * 16);
-#pragma unroll
-        for (int i = 0; i < NA; i++) fa[i] = *reinterpret_cast<const v4i *>(adig + (s & 1) * (NA * 1024) + i * 1024 + lane * 16);
-        if (s + STG < ksteps) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0): the reads above have returned before their stage is overwritten
-            issue(s + STG);
+        for (int z = 0; z < 4; z++) {
+            rb_lo = v[z] < rb_lo ? v[z] : rb_lo;
+            rb_hi = v[z] > rb_hi ? v[z] : rb_hi;
         }
-        // the weights of this step: range, digits
-        int x[16];
+    };
+    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+    const int sh = p.shift;
+    // diagonals of one output -> 128-bit sum -> shift -> C and R (diagonals are added in 64-bit groups of four, the groups
+    // meet in 128 bits)
+    auto finish = [&](const int (&dg)[D], int m, int n) {
+        u128 sum = (u128)(i128)p.init;
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int gq = 0; gq < (D + 3) / 4; gq++) {
+            uint64_t sg = (uint64_t)(int64_t)dg[4 * gq];
 #pragma unroll
-            for (int z = 0; z < 4; z++) {
-                x[4 * j + z] = raw[j][z];
-                rb_lo = raw[j][z] < rb_lo ? raw[j][z] : rb_lo;
-                rb_hi = raw[j][z] > rb_hi ? raw[j][z] : rb_hi;
+            for (int j = 1; j < 4; j++)
+                if (4 * gq + j < D) sg += (uint64_t)(int64_t)dg[4 * gq + j] << (8 * j);
+            sum += (u128)(i128)(int64_t)sg << (32 * gq);
+        }
+        if (!(m < m_lim && n < p.N)) return;
+        const uint64_t lo = (uint64_t)sum, hi = (uint64_t)(sum >> 64);
+        const long o = (long)m * p.ldc + n;
+        p.C[o] = (int64_t)((lo >> sh) | ((hi << 1) << (63 - sh)));
+        if (p.R) p.R[o] = (int64_t)(lo & rmask);
+    };
+
+    if (m_lim - m0 <= 16) {
+        // ---- at most 16 rows (nearly every tile of a routed expert): v_mfma_i32_16x16x64_i8, half the matrix work ----
+        // Lane (i, q) = (lane % 16, lane / 16) of either operand holds k = 16q .. 16q+15 of a pair of steps for row i of
+        // A, or for column 16 ct + i of B (ct = 0, 1: the wavefront's two column tiles).  That is half q % 2 of step
+        // 2u + q / 2: a lane reads at the steps of its own parity only and keeps what it read; the products follow at
+        // the odd steps (and at a last even one, where the lanes of the missing step hold zeros for A).
+        const int li = lane & 15, lq = lane >> 4;
+        const bool odd_lane = (lq >> 1) != 0;
+        int b_rd16[2][4];
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int nn = 16 * ct + li;
+                b_rd16[ct][j] = (nn >> 3) * 1024 + (8 * (nn & 7) + 4 * (lq & 1) + ((j ^ (nn >> 3)) & 3)) * 16;
             }
-        v4i fb[NB];
-        split16_w32<NB>(x, fb);
-        // this wavefront's eighth of A for the next step
-        if (s + 1 < ksteps) stash_a(araw, (s + 1) & 1);
+        const int a_rd16 = (li + 32 * (lq & 1)) * 16;
+        v4i acc[D][2];
 #pragma unroll
-        for (int i = 0; i < NA; i++)
+        for (int d = 0; d < D; d++)
 #pragma unroll
-            for (int j = 0; j < NB; j++)
-                acc[i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i + j], 0, 0, 0);
-        __syncthreads();
+            for (int ct = 0; ct < 2; ct++) acc[d][ct] = v4i{ 0, 0, 0, 0 };
+        v4i raw[2][4], fa[NA];
+#pragma unroll
+        for (int i = 0; i < NA; i++) fa[i] = v4i{ 0, 0, 0, 0 };
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) raw[ct][j] = v4i{ 0, 0, 0, 0 };
+
+        for (int s = 0; s < ksteps; s++) {
+            landed(s);
+            const unsigned st = (unsigned)(s % STG);
+            const bool mine = odd_lane == ((s & 1) != 0);
+            if (mine) {
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) raw[ct][j] = *reinterpret_cast<const v4i *>(ring_b + st * 4096 + b_rd16[ct][j]);
+#pragma unroll
+                for (int i = 0; i < NA; i++) fa[i] = *reinterpret_cast<const v4i *>(adig + (s & 1) * (NA * 1024) + i * 1024 + a_rd16);
+            }
+            const v4i araw = *reinterpret_cast<const v4i *>(ring_a + st * 8192 + wave * 1024 + lane * 16);
+            if (s + STG < ksteps) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0): the reads above have returned before their stage is overwritten
+                issue(s + STG);
+            }
+            if (mine) {
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) track_b(raw[ct][j]);
+            }
+            if (s + 1 < ksteps) stash_a(araw, (s + 1) & 1);
+            const bool last_even = s + 1 == ksteps && !(s & 1);
+            if ((s & 1) || last_even) {
+                if (last_even && odd_lane) {               // no step 2u + 1: these lanes multiply zeros
+#pragma unroll
+                    for (int i = 0; i < NA; i++) fa[i] = v4i{ 0, 0, 0, 0 };
+                }
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) {
+                    int x[16];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int z = 0; z < 4; z++) x[4 * j + z] = raw[ct][j][z];
+                    v4i fb[NB];
+                    split16_w32<NB>(x, fb);
+#pragma unroll
+                    for (int i = 0; i < NA; i++)
+#pragma unroll
+                        for (int j = 0; j < NB; j++)
+                            acc[i + j][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[i], fb[j], acc[i + j][ct], 0, 0, 0);
+                }
+            }
+            __syncthreads();
+        }
+        // accumulator register r of lane l holds row 4 (l / 16) + r, column l % 16 of its column tile
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int dg[D];
+#pragma unroll
+                for (int d = 0; d < D; d++) dg[d] = acc[d][ct][r];
+                finish(dg, m0 + 4 * lq + r, n0 + 16 * ct + li);
+            }
+    } else {
+        v16i acc[D];
+#pragma unroll
+        for (int d = 0; d < D; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[d][r] = 0;
+
+        for (int s = 0; s < ksteps; s++) {
+            landed(s);
+            const unsigned st = (unsigned)(s % STG);
+            v4i raw[4], araw, fa[NA];
+#pragma unroll
+            for (int j = 0; j < 4; j++) raw[j] = *reinterpret_cast<const v4i *>(ring_b + st * 4096 + b_rd[j]);
+            araw = *reinterpret_cast<const v4i *>(ring_a + st * 8192 + wave * 1024 + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NA; i++) fa[i] = *reinterpret_cast<const v4i *>(adig + (s & 1) * (NA * 1024) + i * 1024 + lane * 16);
+            if (s + STG < ksteps) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0): the reads above have returned before their stage is overwritten
+                issue(s + STG);
+            }
+            // the weights of this step: range, digits
+            int x[16];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                track_b(raw[j]);
+#pragma unroll
+                for (int z = 0; z < 4; z++) x[4 * j + z] = raw[j][z];
+            }
+            v4i fb[NB];
+            split16_w32<NB>(x, fb);
+            // this wavefront's eighth of A for the next step
+            if (s + 1 < ksteps) stash_a(araw, (s + 1) & 1);
+#pragma unroll
+            for (int i = 0; i < NA; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i + j], 0, 0, 0);
+            __syncthreads();
+        }
+        // accumulator register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            int dg[D];
+#pragma unroll
+            for (int d = 0; d < D; d++) dg[d] = acc[d][r];
+            finish(dg, m0 + 4 * (lane >> 5) + 8 * (r >> 2) + (r & 3), n0 + (lane & 31));
+        }
     }
 
     // every workgroup leaves its ranges in its own slot; the waves' ranges meet in LDS (the rings are free by now)
@@ -185,31 +313,6 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
         slot[1] = (unsigned long long)ra.hi ^ kSignFlip;
         slot[2] = (unsigned long long)rb.lo ^ kSignFlip;
         slot[3] = (unsigned long long)rb.hi ^ kSignFlip;
-    }
-
-    // epilogue: diagonals -> 128-bit sum -> shift (accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
-    // column l%32; diagonals are added in 64-bit groups of four, the groups meet in 128 bits)
-    const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
-    const int sh = p.shift;
-    const int n = n0 + (lane & 31);
-    const int mrow = m0 + 4 * (lane >> 5);
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int dr = 8 * (r >> 2) + (r & 3);
-        u128 sum = (u128)(i128)p.init;
-#pragma unroll
-        for (int gq = 0; gq < (D + 3) / 4; gq++) {
-            uint64_t sg = (uint64_t)(int64_t)acc[4 * gq][r];
-#pragma unroll
-            for (int j = 1; j < 4; j++)
-                if (4 * gq + j < D) sg += (uint64_t)(int64_t)acc[4 * gq + j][r] << (8 * j);
-            sum += (u128)(i128)(int64_t)sg << (32 * gq);
-        }
-        if (!(mrow + dr < m_lim && n < p.N)) continue;
-        const uint64_t lo = (uint64_t)sum, hi = (uint64_t)(sum >> 64);
-        const long o = (long)(mrow + dr) * p.ldc + n;
-        p.C[o] = (int64_t)((lo >> sh) | ((hi << 1) << (63 - sh)));
-        if (p.R) p.R[o] = (int64_t)(lo & rmask);
     }
 }
 
