@@ -10,9 +10,12 @@
 #include <vector>
 
 // Tuning knobs: MFMA depths (32 k each) per pipeline step by diagonal count, and how many vector-ALU
-// instructions of the digit split are scheduled behind each MFMA of a step's last depth.
+// instructions of the digit split are scheduled behind each MFMA of a step's last depth.  (A 32x32x32 MFMA holds the
+// matrix pipe for 32 cycles, a vector instruction its own for 4; with two wavefronts on a SIMD up to four or five
+// vector instructions per MFMA run in its shade, eight cost a quarter more time per MFMA: measured with a probe, and
+// on the 512 x 7168 x 18432 product 0.631-0.638 ms with 5 against 0.642-0.643 with 8.)
 #ifndef ZK_VALU_PER_MFMA
-#define ZK_VALU_PER_MFMA 8
+#define ZK_VALU_PER_MFMA 5
 #endif
 #ifndef ZK_KK
 #define ZK_KK(DD) 1
