@@ -557,6 +557,61 @@ def test_einsums_model_shapes(K, oracle, path):
     assert np.array_equal(host(x), oracle.einsum_bshc_hdc_bshd(host(o), wkv_b_2, 31))
 
 
+def test_empty_operands(K, oracle):
+    """operands without elements, as torch hands them over (null data pointers): no rows, columns or batches is a call
+    that does nothing; an empty contraction leaves the rounding term shifted in every output, as the reference's loop
+    over no elements does (int64_gemm.cu:44-78), for the two products, the einsums and the grouped launch; softmax,
+    activations, RMSNorm, RoPE and the dispatch of no tokens return without an error"""
+    z = lambda *shape, dtype=torch.int64: torch.zeros(shape, dtype=dtype, device="cuda")
+    ones = lambda *shape: torch.ones(shape, dtype=torch.int64, device="cuda")
+    for A, W in ((z(1, 0, 64), ones(8, 64)), (ones(1, 4, 64), z(0, 64)), (z(0, 4, 64), ones(8, 64))):
+        C, R = K.int64_bmm_broadcast(A, W, 1, 1, 3)
+        assert C.numel() == 0 and R.numel() == 0
+    for path in (0, 1, 2):
+        K.lib.zk_gemm_set_path(path)
+        try:
+            for M, N, w32, c in ((4, 8, False, 3), (200, 300, False, 0), (5, 7, True, 63), (16, 576, True, 17)):
+                C = torch.full((2, M, N), 77, dtype=torch.int64, device="cuda")
+                R = torch.full((2, M, N), 77, dtype=torch.int64, device="cuda")
+                A, W = z(2, M, 0), z(N, 0, dtype=torch.int32 if w32 else torch.int64)
+                fn = K.lib.int64_32_bmm_broadcast_launcher if w32 else K.lib.int64_64_bmm_broadcast_launcher
+                fn(A.data_ptr(), W.data_ptr(), C.data_ptr(), R.data_ptr(), 1, 1, c, 2, M, 0, N)
+                K._check("bmm with K = 0")
+                Ce, Re = oracle.int64_bmm_broadcast(np.zeros((2, M, 0), np.int64), np.zeros((N, 0), np.int64), 1, 1, c)
+                assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re), (path, M, N, w32, c)
+        finally:
+            K.lib.zk_gemm_set_path(0)
+    for rescale in (0, 1, 7, 40):
+        o = K.einsum_bshd_hdc_bshc(z(1, 2, 3, 0), z(3, 0, 5, dtype=torch.int32), rescale)
+        assert np.array_equal(host(o), oracle.einsum_bshd_hdc_bshc(np.zeros((1, 2, 3, 0), np.int64), np.zeros((3, 0, 5), np.int32), rescale))
+        o = K.einsum_bshc_btc_bsht(z(1, 2, 3, 0), z(1, 4, 0), rescale)
+        assert np.array_equal(host(o), oracle.einsum_bshc_btc_bsht(np.zeros((1, 2, 3, 0), np.int64), np.zeros((1, 4, 0), np.int64), rescale))
+        o = K.einsum_bsht_btc_bshc(z(1, 2, 3, 0), z(1, 0, 8), rescale)
+        assert np.array_equal(host(o), oracle.einsum_bsht_btc_bshc(np.zeros((1, 2, 3, 0), np.int64), np.zeros((1, 0, 8), np.int64), rescale))
+        o = K.einsum_bshc_hdc_bshd(z(1, 2, 3, 0), z(3, 6, 0, dtype=torch.int32), rescale)
+        assert np.array_equal(host(o), oracle.einsum_bshc_hdc_bshd(np.zeros((1, 2, 3, 0), np.int64), np.zeros((3, 6, 0), np.int32), rescale))
+    assert K.einsum_bshc_btc_bsht(ones(1, 2, 3, 8), z(1, 0, 8), 7).shape == (1, 2, 3, 0)
+    # the grouped launch over an empty contraction
+    idx = dev(np.array([[0, 2], [1, 2], [2, 0]], dtype=np.int64))
+    d = K.moe_dispatch(idx, 4)
+    ws = [z(6, 0, dtype=torch.int32) for _ in range(4)]
+    table = torch.tensor([0x1000 * (i + 1) for i in range(4)], dtype=torch.int64, device="cuda")   # (never dereferenced)
+    del ws
+    C, R = K.int64_grouped_bmm(z(6, 0), table, True, 6, 5, d, want_remainder=True)
+    assert not host(C).any() and not host(R).any()
+    # the kernels that are no products
+    K.softmax_init_q19(); K.softmax_init_q21(); K.silu_init_q23(); K.silu_init_q25()
+    for fn, shape in ((K.softmax_q19, (1, 0, 4, 16)), (K.softmax_q19, (1, 2, 4, 0)), (K.softmax_q21, (0, 2, 4, 16)),
+                      (K.silu_q23, (1, 0, 16)), (K.sigmoid_q23, (0, 3, 16)), (K.silu_q25, (2, 3, 0)), (K.sigmoid_q25, (1, 0, 0))):
+        Rz = z(*shape)
+        fn(Rz, torch.empty_like(Rz))
+    out, _ = K.RMS_Norm_int64(z(0, 64), ones(64), 10, 64)
+    assert out.shape == (0, 64)
+    assert K.complex_int64_mul_broadcast(z(1, 0, 4, 8, 2), z(0, 8, 2)).numel() == 0
+    d0 = K.moe_dispatch(z(0, 8), 16)
+    assert int(d0["ntiles"].item()) == 0 and not host(d0["seg"]).any()
+
+
 # ---------------------------------------------------------------------------------- softmax -----
 def test_einsum_values_rewritten_with_contiguous_rows(K, oracle, monkeypatch):
     """`bsht,btc->bshc` on the MFMA path copies a small n-contiguous int64 B into row-major scratch first (products of

@@ -12,8 +12,32 @@ static int g_last_path = 0, g_last_la = 0, g_last_lb = 0;
 static bool g_last_digits = false;      // the last call ran on kernels with fixed digit counts (gemm_mfma.hip), whose plan and planes are reported
 static long g_grouped_mfma_calls = 0;
 
+// An empty contraction (K == 0): every output is the rounding term shifted, as the reference's loop over no elements leaves
+// it (int64_gemm.cu:44-78); A and B hold nothing and are never read.
+static __global__ void gemm_empty_k_kernel(int64_t *C, int64_t *R, long ldc, long sC, int M, int N, long total, int64_t quotient, int64_t remainder)
+{
+    for (long o = (long)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (long)gridDim.x * blockDim.x) {
+        const long g = o / ((long)M * N), r = o - g * ((long)M * N);
+        const long at = g * sC + (r / N) * ldc + r % N;
+        C[at] = quotient;
+        if (R) R[at] = remainder;
+    }
+}
+
+static bool gemm_empty_k(const char *name, int64_t *C, int64_t *R, long ldc, long sC, int G, int M, int N, int shift, int64_t init)
+{
+    const long total = (long)G * M * N;
+    if (total == 0) return true;
+    const int64_t mask = shift ? (int64_t)(((uint64_t)1 << shift) - 1) : 0;
+    const long blocks = (total + 255) / 256;
+    gemm_empty_k_kernel<<<dim3((unsigned)(blocks < 4096 ? blocks : 4096)), 256, 0, 0>>>(C, R, ldc, sC, M, N, total, init >> shift, init & mask);
+    g_last_path = kPathValu; g_last_la = 0; g_last_lb = 0; g_last_digits = false;
+    return check_launch(name);
+}
+
 bool gemm_dispatch(const char *name, const GemmDesc &d)
 {
+    if (d.K == 0) return gemm_empty_k(name, d.C, d.R, d.ldc, d.sC, d.G, d.M, d.N, d.shift, d.init);
     // one or two rows (a decoding step, the head): the exact vector-ALU stream over the weights, unless the MFMA
     // path is asked for by name
     // (prepared weights: the MFMA kernels read a few bytes per weight where the matrix-vector stream reads eight, so
@@ -62,6 +86,7 @@ constexpr int kGroupedGemvMaxRows = 64;
 
 void gemm_grouped_dispatch(const char *name, const GroupedDesc &d)
 {
+    if (d.K == 0) { gemm_empty_k(name, d.C, d.R, d.ldc, 0, 1, d.rows, d.N, d.shift, d.init); return; }
     // (prepared weights: from 33 rows on the MFMA kernels first, as in gemm_dispatch; below that the handful of tiles
     // leaves most of the device idle and the row-by-row stream is faster: one token 0.52 against 0.66 ms)
     const bool prepared = g_gemm_path != kPathValu && !d.b32 && d.rows > 32 && gemm_mfma_is_prepared((const void *)d.B);
@@ -138,7 +163,7 @@ static void bmm(const char *name, const int64_t *A, const void *B, int b32, int6
     if (!dims_ok(name, { Bdim, M, K, N }, c_rs)) return;
     if (a_rs == 0 || b_rs == 0) { set_error(kBadArgument, "%s: zero rescale divisor", name); return; }
     if ((long)Bdim * M * N == 0) return;
-    if (!A || !B || !C) { set_error(kBadArgument, "%s: null pointer", name); return; }
+    if (((!A || !B) && K > 0) || !C) { set_error(kBadArgument, "%s: null pointer", name); return; }
     GemmDesc d;
     d.A = A; d.lda = K; d.sA = (long)M * K;
     d.B = B; d.b32 = b32; d.ldbn = K; d.ldbk = 1; d.sB = 0;
@@ -173,7 +198,7 @@ void einsum_bshd_hdc_bshc(const int64_t *q_nope, const int32_t *wkv_b_1, int64_t
     const char *name = "einsum_bshd_hdc_bshc";
     if (!zk::dims_ok(name, { B, S, H, D, C }, rescale)) return;
     if ((long)B * S * H * C == 0) return;
-    if (!q_nope || !wkv_b_1 || !out) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    if (((!q_nope || !wkv_b_1) && D > 0) || !out) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
     zk::GemmDesc d;
     d.A = q_nope; d.lda = (long)H * D; d.sA = D;
     d.B = wkv_b_1; d.b32 = 1; d.ldbn = 1; d.ldbk = C; d.sB = (long)D * C;
@@ -190,7 +215,7 @@ void einsum_bshc_btc_bsht(const int64_t *A, const int64_t *B, int64_t *C, int64_
     const char *name = "einsum_bshc_btc_bsht";
     if (!zk::dims_ok(name, { Bsz, S, H, T, Cdim }, rescale)) return;
     if ((long)Bsz * S * H * T == 0) return;
-    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    if (((!A || !B) && Cdim > 0) || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
     zk::GemmDesc d;
     d.A = A; d.lda = Cdim; d.sA = (long)S * H * Cdim;
     d.B = B; d.b32 = 0; d.ldbn = Cdim; d.ldbk = 1; d.sB = (long)T * Cdim;
@@ -207,7 +232,7 @@ void einsum_bsht_btc_bshc(const int64_t *A, const int64_t *B, int64_t *C, int64_
     const char *name = "einsum_bsht_btc_bshc";
     if (!zk::dims_ok(name, { Bsz, S, H, T, Cdim }, rescale)) return;
     if ((long)Bsz * S * H * Cdim == 0) return;
-    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    if (((!A || !B) && T > 0) || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
     zk::GemmDesc d;
     d.A = A; d.lda = T; d.sA = (long)S * H * T;
     d.B = B; d.b32 = 0; d.ldbn = 1; d.ldbk = Cdim; d.sB = (long)T * Cdim;
@@ -224,7 +249,7 @@ void einsum_bshc_hdc_bshd(const int64_t *A, const int32_t *B, int64_t *C, int64_
     const char *name = "einsum_bshc_hdc_bshd";
     if (!zk::dims_ok(name, { Bsz, S, H, D, Cdim }, rescale)) return;
     if ((long)Bsz * S * H * D == 0) return;
-    if (!A || !B || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    if (((!A || !B) && Cdim > 0) || !C) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
     zk::GemmDesc d;
     d.A = A; d.lda = (long)H * Cdim; d.sA = Cdim;
     d.B = B; d.b32 = 1; d.ldbn = Cdim; d.ldbk = 1; d.sB = (long)D * Cdim;

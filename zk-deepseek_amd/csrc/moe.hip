@@ -144,7 +144,7 @@ void moe_dispatch(const int64_t *indices, int T, int K, int E, int *counts_scrat
 {
     const char *name = "moe_dispatch";
     if (T < 0 || K <= 0 || E <= 0) { zk::set_error(zk::kBadArgument, "%s: bad dimension", name); return; }
-    if (!indices || !counts_scratch || !seg || !sorted_token || !sorted_pos || !tiles || !ntiles) {
+    if (((!indices || !sorted_token || !sorted_pos) && T > 0) || !counts_scratch || !seg || !tiles || !ntiles) {
         zk::set_error(zk::kBadArgument, "%s: null pointer", name);
         return;
     }
@@ -196,7 +196,7 @@ void int64_grouped_bmm_launcher(const int64_t *A, const void *const *B_ptrs, int
     const char *name = "int64_grouped_bmm_launcher";
     if (groups < 0 || rows < 0 || K < 0 || N < 0 || c_rescale < 0 || c_rescale > 63) { zk::set_error(zk::kBadArgument, "%s: bad argument", name); return; }
     if (groups == 0 || rows == 0 || N == 0) return;
-    if (!A || !B_ptrs || !C || !seg || !tiles || !ntiles) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
+    if ((!A && K > 0) || !B_ptrs || !C || !seg || !tiles || !ntiles) { zk::set_error(zk::kBadArgument, "%s: null pointer", name); return; }
     zk::GroupedDesc d;
     d.A = A; d.lda = K; d.B = B_ptrs; d.b32 = b32; d.C = C; d.R = R; d.ldc = N;
     d.seg = seg; d.tiles = tiles; d.ntiles = ntiles;
