@@ -10,9 +10,9 @@ from util import rand_i32, rand_i64
 
 pytestmark = pytest.mark.gpu
 
-# ZK_TEST_SEEDS=n multiplies the seed ranges of the three randomly drawn problem sets below (40, 20 and 10 seeds by
+# ZK_TEST_SEEDS=n multiplies the seed ranges of the randomly drawn problem sets below (40, 20, 10 and 10 seeds by
 # default), e.g. `ZK_TEST_SEEDS=200 python -m pytest tests/test_gpu_parity.py -m gpu -x -q -k seeded_random` runs 8000 +
-# 4000 + 2000 seeds and stops at the first mismatch
+# 4000 + 2000 + 2000 seeds and stops at the first mismatch
 SEEDS = max(1, int(os.environ.get("ZK_TEST_SEEDS", "1") or 1))
 
 
@@ -1406,6 +1406,46 @@ def test_int64_grouped_bmm_int32_weights_streamed_odd_operands(K, oracle, monkey
     finally:
         monkeypatch.delenv("ZK_STREAM32_MIN_PAIRS", raising=False)
         K.lib.zk_reload_env()
+
+
+@pytest.mark.parametrize("seed", range(10 * SEEDS))
+def test_grouped_bmm_seeded_random_problems(K, oracle, seed):
+    """the grouped launch on randomly drawn routings, shapes, operand widths, weight types and shifts: experts without
+    rows, with a handful and with several tiles' worth; whole and ragged steps of K (the streamed int32 kernel takes the
+    former), ragged tile columns; a few rows in all (the matrix-vector kernels) or many; digits the 32-row kernels
+    hold or not (the 16-row kernels behind them); every problem twice, the second call on what the first one learnt"""
+    rng = np.random.default_rng(9900 + seed)
+    for _ in range(4):
+        T = int(rng.choice([1, 3, 8, 40, 150, 400]))
+        E = int(rng.choice([2, 8, 16, 40]))
+        Kr = int(rng.choice([1, 2, 4]))
+        Kr = min(Kr, E)
+        Kd = int(rng.choice([32, 64, 96, 160, 200, 224, 520]))
+        N = int(rng.choice([16, 64, 250, 256, 300, 700]))
+        while T * Kr * Kd * N > 80_000_000:
+            T = max(1, T // 2)
+        w32 = bool(rng.integers(0, 3))
+        bits_a = int(rng.choice([12, 20, 28, 31, 37, 47, 60]))
+        bits_w = int(rng.choice([12, 16, 24, 28, 31])) if w32 else int(rng.choice([16, 24, 33, 50]))
+        c = int(rng.choice([0, 8, 17, 23, 31, 40]))
+        idx = _routing(rng, T, E, Kr)
+        if T >= 40 and rng.integers(0, 2):
+            idx[: T // 2, 0] = int(idx[0, 0])                # one expert with several tiles
+            for t in range(T // 2):
+                others = [e for e in rng.permutation(E) if e != idx[t, 0]][: Kr - 1]
+                idx[t, 1:] = others
+        x = rand_i64(rng, (T, Kd), bits_a)
+        ws = [rand_i32(rng, (N, Kd), bits_w) if w32 else rand_i64(rng, (N, Kd), bits_w) for _ in range(E)]
+        d = K.moe_dispatch(dev(idx), E)
+        xs = K.moe_gather_rows(dev(x), d)
+        seg, tok, _ = oracle.moe_dispatch(idx, E)
+        wd = [dev(w) for w in ws]
+        table = K.pointer_table(wd)
+        Ce, Re = oracle.grouped_bmm(x[tok], ws, seg, c)
+        for rep in range(2):
+            C, R = K.int64_grouped_bmm(xs, table, w32, N, c, d, want_remainder=True)
+            ok = np.array_equal(host(C), Ce) and np.array_equal(host(R), Re)
+            assert ok, "T=%d E=%d Kr=%d K=%d N=%d w32=%s bits=(%d,%d) c=%d call %d plan %s" % (T, E, Kr, Kd, N, w32, bits_a, bits_w, c, rep, K.gemm_last_plan())
 
 
 @pytest.mark.parametrize("w32", [False, True])
