@@ -362,19 +362,20 @@ def test_stale_guess_divided_weights(K, oracle, w32):
     _stale_guess_rounds(K, _bmm(K, A, W, 29, 1, 256), lambda: oracle.int64_bmm_broadcast(A.h, W.h, 1, 256, 29), [A, W], pokes)
 
 
-@pytest.mark.parametrize("w32", [False, True])
-def test_stale_guess_grouped_launch(K, oracle, w32):
+@pytest.mark.parametrize("w32,bits", [(False, (20, 16)), (True, (20, 16)), (True, (28, 28))])
+def test_stale_guess_grouped_launch(K, oracle, w32, bits):
     """the routed experts' grouped product: activations gathered into a buffer of their own for every call, weights seen
     before.  Once the weights are known the launch does not wait for its verdict; a guarded launch of the 16-row
     kernels behind it computes everything again when the digits guessed from the last activations (or remembered for
-    the weights) were too few."""
-    rng = np.random.default_rng(40 + w32)
+    the weights) were too few.  (28, 28)-bit operands on int32 weights are sixteen digit pairs: the launch that streams the
+    weights through LDS rings, whose tiles of at most 16 rows track what they load in their own way."""
+    rng = np.random.default_rng(40 + w32 + bits[0])
     T, E, Kr, Kd, N = 150, 10, 4, 192, 520
     idx = np.stack([rng.permutation(E)[:Kr] for _ in range(T)]).astype(np.int64)
     idx[:50, 0] = 3                                  # one expert with more than a tile of rows
     idx[:50, 1:] = np.stack([rng.permutation([0, 1, 2, 4, 5, 6])[: Kr - 1] for _ in range(50)])
-    X = Operand(rand_i64(rng, (T, Kd), 20))
-    Ws = [Operand(rand_i32(rng, (N, Kd), 16) if w32 else rand_i64(rng, (N, Kd), 16)) for _ in range(E)]
+    X = Operand(rand_i64(rng, (T, Kd), bits[0]))
+    Ws = [Operand(rand_i32(rng, (N, Kd), bits[1]) if w32 else rand_i64(rng, (N, Kd), bits[1])) for _ in range(E)]
     table = K.pointer_table([w.d for w in Ws])
     d = K.moe_dispatch(torch.from_numpy(idx).cuda(), E)
     seg, tok, _ = oracle.moe_dispatch(idx, E)
@@ -387,10 +388,14 @@ def test_stale_guess_grouped_launch(K, oracle, w32):
 
     # (four digits where there were three: the 32-row kernels have instances for that; beyond five digits the product
     #  would move to the 16-row kernels altogether)
-    wide = 1 << 29
+    wide, wide_w = (1 << 29, 1 << 29) if bits[0] == 20 else (1 << 36, (1 << 31) - 1)       # (a fifth digit where there were four)
+    streamed = K.lib.zk_gemm_grouped_streamed_calls()
     pokes = [lambda: X.poke((0, 0), wide), lambda: X.poke((T - 1, Kd - 1), -wide), lambda: X.poke((row_of_busiest, 77), wide),
-             lambda: Ws[busiest].poke((N - 1, Kd - 1), -wide), lambda: Ws[int(idx[T - 1, 0])].poke((0, 0), wide)]
+             lambda: Ws[busiest].poke((N - 1, Kd - 1), -wide_w if bits[0] == 20 else wide_w),      # (no negative int32 needs a fifth digit)
+             lambda: Ws[int(idx[T - 1, 0])].poke((0, 0), wide_w)]
     _stale_guess_rounds(K, call, lambda: oracle.grouped_bmm(X.h[tok], [w.h for w in Ws], seg, 19), [X] + Ws, pokes)
+    if bits[0] == 28:
+        assert K.lib.zk_gemm_grouped_streamed_calls() - streamed >= 5 * 4, "the launches under test were to run on the streamed kernel"
 
 
 def test_declined_product_runs_although_an_older_error_is_pending(K, oracle):
