@@ -892,7 +892,7 @@ int gemm_mfma_grouped(const GroupedDesc &d, int *limbs_a, int *limbs_b)
         if (pairs * ksteps * 32 * 16384 > 0x7FFFFFFFL) return 1;
         p.tiles_n = (d.N + inst->bn - 1) / inst->bn;
         const long max_mtiles = (long)d.rows / 32 + d.groups;
-        const long blocks = max_mtiles * p.tiles_n;
+        const long blocks = (max_mtiles + 7) / 8 * 8 * p.tiles_n;       // (whole rounds of the 8 XCDs: see the kernels' tile order)
         if (blocks > 0x7FFFFFFFL / 8) return 1;
         p.main_tiles = (int)blocks;
         if (const Outcome got = grow(g_cache.wg, g_cache.wg_count, (size_t)blocks * 4, "range slots")) return got;

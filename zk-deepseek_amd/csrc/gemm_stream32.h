@@ -39,13 +39,15 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
     unsigned char *adig = ring_a + STG * 8192;                               // [2][digit][1 KB], fragment order
     const unsigned ring_b_lds = (unsigned)(uintptr_t)ring_b, ring_a_lds = (unsigned)(uintptr_t)ring_a + wave * 1024;
 
-    const int mt = (int)blockIdx.x / p.tiles_n;
+    // (the tile columns of one 32-row tile on one XCD, as in gemm_mfma_block's grouped form: its rows of A come from memory once)
+    const int xcd = (int)blockIdx.x & 7, w = (int)blockIdx.x >> 3, wq = w / p.tiles_n;
+    const int mt = wq * 8 + xcd;
     unsigned long long *slot = p.wg_range + 4 * (long)blockIdx.x;
     if (mt >= *p.grp_ntiles) {                   // the grid covers the worst case: nothing to do, an empty range
         if (tid == 0) { slot[0] = ~0ull; slot[1] = 0ull; slot[2] = ~0ull; slot[3] = 0ull; }
         return;
     }
-    const int tn = (int)blockIdx.x - mt * p.tiles_n;
+    const int tn = w - wq * p.tiles_n;
     const int e = p.grp_tiles[2 * mt];
     const int m0 = p.grp_tiles[2 * mt + 1], m_lim = p.grp_seg[e + 1];
     const int32_t *b_base = reinterpret_cast<const int32_t *>(p.grp_b[e]);
