@@ -839,6 +839,10 @@ def run():
     for nm in ("moe_experts_int32_256tok_top8_of_256", "moe_experts_config5_256tok_top8_of_256"):
         if nm in extra:
             flat[nm + "_frac_hbm"] = extra[nm]["frac_hbm_peak"]
+    if "moe_experts_int32_256tok_top8_of_256" in extra:
+        # (counter traffic of the layer's three grouped launches against their algorithmic bytes, from the committed profile)
+        flat["moe_experts_int32_gemm_traffic"] = measured_traffic("moe_experts_int32_gemm_bytes_per_call")
+        flat["moe_experts_int32_gemm_algorithmic_bytes"] = measured_traffic("moe_experts_int32_gemm_algorithmic_bytes_per_call")
     roofline.update(flat)
     roofline["others"] = others
     cold = {}
