@@ -17,6 +17,10 @@
 // and lane l lands at byte 16 l of the instruction's 1 KB block.  Lane 8r + c of instruction q loads chunk
 // (c & 4) | ((c ^ q) & 3) of row 8q + r, so chunk 4h + j of row n sits at slot 8 (n % 8) + 4h + (j ^ (n / 8)) of block
 // n / 8: for a fixed j the 64 lanes of a read hit 64 different slots.
+//
+// Tiles of at most 16 rows (nearly every tile of a routed expert) multiply on v_mfma_i32_16x16x64_i8 over pairs of steps:
+// half the matrix work for the same bytes, which on this power-managed device is what lets the stream run faster.  For
+// the same reason rows past the end of a segment are multiplied as zeros, not as copies of its last row.
 #pragma once
 #include "lds_dma.h"
 
