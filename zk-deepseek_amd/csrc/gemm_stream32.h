@@ -57,9 +57,9 @@ __global__ __launch_bounds__(512) void gemm_stream32_grouped_kernel(MfmaParams p
     const int32_t *b_base = reinterpret_cast<const int32_t *>(p.grp_b[e]);
     if ((uintptr_t)b_base & 15) {
         // a matrix that does not start on a 16-byte boundary: the loads into LDS cannot take it.  The workgroup reports
-        // the full range instead of computing: no digit count covers that, so the guarded launch behind this one (or
-        // the caller's next route) computes these outputs.
-        if (tid == 0) { slot[0] = 0ull; slot[1] = ~0ull; slot[2] = 0ull; slot[3] = ~0ull; }
+        // the full range for B instead of computing (and nothing for A, which it has not looked at): no digit count
+        // covers that, so the guarded launch behind this one (or the caller's next route) computes these outputs.
+        if (tid == 0) { slot[0] = ~0ull; slot[1] = 0ull; slot[2] = 0ull; slot[3] = ~0ull; }
         return;
     }
     const int n0 = tn * 256 + wave * 32;
