@@ -245,6 +245,9 @@ long zk_gemm_grouped_mfma_calls(void);
 /* How many of those launches ran on the kernel that streams int32 weights through LDS rings (K a multiple of 32,
  * sixteen digit pairs or more; ZK_STREAM32_MIN_PAIRS and ZK_NO_STREAM32 move or remove that choice). */
 long zk_gemm_grouped_streamed_calls(void);
+/* How many GEMM launches so far ran on the software-pipelined 128 x 128 kernel that reads digit planes on both sides
+ * (weights prepared with zk_gemm_prepare_weights, three digits a side; ZK_NO_PIPE=1 switches it off). */
+long zk_gemm_pipe_calls(void);
 /* No reference counterpart: model weights do not change between calls, so a weight matrix W[N,K] (int64, or int32 with
  * b32 != 0; groups == 0, B = the device pointer later passed as B) or all the matrices of a device table of pointers
  * (groups > 0, B = the table later passed to int64_grouped_bmm_launcher) can be split into base-256 digit planes ONCE.

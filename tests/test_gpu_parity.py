@@ -376,6 +376,36 @@ def test_gemm_prepared_weights(K, oracle, bits_w):
         assert K.lib.zk_gemm_last_prepared() == 0
 
 
+def test_gemm_prepared_weights_pipelined_kernel(K, oracle):
+    """three digits a side with planes for both operands run on the software-pipelined 128 x 128 kernel (loads through a
+    ring of LDS stages, the next step's fragments read beside the MFMAs): several rounds of tiles with the last one cut
+    along K, a K that is not a whole step and one shorter than the ring is deep, two batches, ragged M and N, int32
+    weights, a K beyond one pass of the int32 accumulators (every tile cut), C alone"""
+    rng = np.random.default_rng(77)
+    keep = []
+    for (Bd, M, N, Kd, bits_a, bits_w, w32, c) in ((1, 640, 6656, 2048, 20, 16, False, 17), (1, 512, 8192, 96, 20, 16, False, 0),
+                                                   (1, 600, 6700, 227, 21, 16, False, 23), (2, 384, 5632, 160, 20, 16, False, 9),
+                                                   (1, 640, 6656, 1024, 20, 16, True, 17), (1, 130, 200, 40, 21, 16, False, 23),
+                                                   (1, 130, 256, 50000, 20, 16, False, 29), (1, 1100, 33000, 100, 20, 16, False, 29)):
+        A = rand_i64(rng, (Bd, M, Kd), bits_a)
+        W = rand_i32(rng, (N, Kd), bits_w) if w32 else rand_i64(rng, (N, Kd), bits_w)
+        Ce, Re = oracle.int64_bmm_broadcast(A, W, 1, 1, c)
+        Ad, Wd = dev(A), dev(W)
+        keep.append(Wd)
+        K.prepare_weights(Wd)
+        try:
+            for rep in range(3):            # (the first call may run on a guess made for other activations at this address)
+                before = K.lib.zk_gemm_pipe_calls()
+                C, R = K.int64_bmm_broadcast(Ad, Wd, 1, 1, c)
+                assert np.array_equal(host(C), Ce) and np.array_equal(host(R), Re), (Bd, M, N, Kd, w32, c, rep)
+            assert K.gemm_last_plan()[1:] == (3, 3) and K.lib.zk_gemm_last_prepared() == 1
+            assert K.lib.zk_gemm_pipe_calls() == before + 1, (Bd, M, N, Kd)
+            C, R = K.int64_bmm_broadcast(Ad, Wd, 1, 1, c, want_remainder=False)
+            assert R is None and np.array_equal(host(C), Ce)
+        finally:
+            K.release_weights(Wd)
+
+
 @pytest.mark.parametrize("w32", [False, True])
 @pytest.mark.parametrize("T,Kr", [(1, 8), (40, 3), (300, 4)])
 def test_grouped_bmm_prepared_weights(K, oracle, T, Kr, w32):

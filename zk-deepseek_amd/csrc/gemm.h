@@ -60,6 +60,7 @@ bool gemm_mfma_is_prepared(const void *B);
 int gemm_mfma_last_pairs();       // digit pairs multiplied per element of K by the last MFMA launch
 int gemm_mfma_last_prepared();    // 1 when the last MFMA launch read B from prepared planes
 long gemm_mfma_grouped_streamed_calls();   // grouped launches so far that ran on the streamed int32 kernel
+long gemm_mfma_pipe_calls();               // launches so far that ran on the software-pipelined kernel for planes on both sides
 
 // Grouped product: the rows of A and C form one contiguous segment per group and every group has its own
 // k-contiguous B[N,K] (the experts of a MoE layer after the tokens have been sorted by expert):

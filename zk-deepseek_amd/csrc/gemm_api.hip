@@ -279,6 +279,7 @@ int zk_gemm_last_pairs(void) { return zk::g_last_digits ? zk::gemm_mfma_last_pai
 
 long zk_gemm_grouped_mfma_calls(void) { return zk::g_grouped_mfma_calls; }
 long zk_gemm_grouped_streamed_calls(void) { return zk::gemm_mfma_grouped_streamed_calls(); }
+long zk_gemm_pipe_calls(void) { return zk::gemm_mfma_pipe_calls(); }
 
 int zk_gemm_last_prepared(void) { return zk::g_last_digits ? zk::gemm_mfma_last_prepared() : 0; }
 int zk_gemm_prepare_weights(const void *B, int b32, int groups, int N, int K) { return zk::gemm_mfma_prepare(B, b32, groups, N, K); }

@@ -33,6 +33,10 @@
 
 namespace zk {
 
+// the 128 x 128 kernel for digit planes on both sides (gemm_mfma_pipe.h), by digit counts (or null), and its dynamic LDS
+MfmaKernel pipe_kernel(int na, int nb);
+size_t pipe_lds_size(int na, int nb);
+
 // the streamed form of the grouped launch for int32 weights (gemm_stream32.h), by digit counts; null: none
 MfmaKernel stream32_grouped_kernel(int na, int nb, size_t *lds);
 MfmaKernel stream32_grouped_kernel_wide(int na, int nb, size_t *lds);
@@ -154,7 +158,7 @@ static RangeCache g_cache;
 // 32-row kernel; ZK_B_ROWS_MIN_MACS: product
 // size from which a small n-contiguous int64 B is rewritten with contiguous rows first; ZK_SKINNY_MAX_M: rows up to
 // which the 32-row tiles are used.
-struct Switches { bool sync_verdict, no_tail_split, valu_fallback, no_stream32; double b_rows_min_macs; int skinny_max_m, planes_min_tiles_n, stream32_min_pairs; };
+struct Switches { bool sync_verdict, no_tail_split, valu_fallback, no_stream32, no_pipe; double b_rows_min_macs; int skinny_max_m, planes_min_tiles_n, stream32_min_pairs; };
 constexpr long kBRowsMinMacs = 1L << 32;
 constexpr double kShapeGuessMaxMacs = 17179869184.0;        // 2^34: about 0.15 ms on the matrix pipe
 // Rows up to which a product runs on the 32-row tiles (two of them from 33 rows on): measured against the 128-row tiles,
@@ -167,6 +171,7 @@ static Switches read_switches()
     s.no_tail_split = getenv("ZK_NO_TAIL_SPLIT") != nullptr;
     s.valu_fallback = getenv("ZK_VALU_FALLBACK") != nullptr;
     s.no_stream32 = getenv("ZK_NO_STREAM32") != nullptr;
+    s.no_pipe = getenv("ZK_NO_PIPE") != nullptr;
     const char *sp = getenv("ZK_STREAM32_MIN_PAIRS");
     s.stream32_min_pairs = sp ? atoi(sp) : 16;
     const char *m = getenv("ZK_B_ROWS_MIN_MACS");
@@ -227,10 +232,11 @@ static void drain_pending()
 }
 
 static int g_last_pairs = 0, g_last_prepared = 0;
-static long g_streamed_calls = 0;
+static long g_streamed_calls = 0, g_pipe_calls = 0;
 int gemm_mfma_last_pairs() { return g_last_pairs; }
 int gemm_mfma_last_prepared() { return g_last_prepared; }
 long gemm_mfma_grouped_streamed_calls() { return g_streamed_calls; }
+long gemm_mfma_pipe_calls() { return g_pipe_calls; }
 
 long gemm_mfma_guard_hits()
 {
@@ -675,6 +681,12 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
                                    : (d.b32 ? (use_planes ? kB32Planes : kB32Fly) : (use_planes ? kB64Planes : kB64Fly));
         MfmaKernel fn = inst->fn[variant];
         if (!fn) return kDeclined;
+        // planes on both sides and the 128 x 128 tile: the software-pipelined form (gemm_mfma_pipe.h; same tiles, planes,
+        // partial sums and outputs)
+        size_t pipe_lds = 0;
+        if (variant == kB64PlanesBoth && !g_switches.no_pipe && BM == 128 && BN == 128 && inst->kk == 1) {
+            if (MfmaKernel pfn = pipe_kernel(inst->na, inst->nb)) { fn = pfn; pipe_lds = pipe_lds_size(inst->na, inst->nb); }
+        }
 
         // Split-K: a launch smaller than the device is cut into `split` slices of K per tile, each a workgroup of
         // its own; with more tiles than compute units the same is done for the tiles of the last, partial round
@@ -759,7 +771,7 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
             // (the owned-k pattern of the planes of A follows the kernel that reads them: prepared planes of B go with the int64 forms)
             inst->planes[(d.b32 && !prep) ? 1 : 0]<<<pgrid, dim3(256), 0, 0>>>(p, g_cache.planes, msub, ksteps, g_cache.mm);
         }
-        const size_t lds = 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
+        const size_t lds = pipe_lds ? pipe_lds : 2 * (size_t)inst->kk * ((BM / 32) * inst->na + (BN / 32) * inst->nb) * 1024 + 9 * 1024 + 16;
         static std::set<const void *> lds_raised;
         if (lds > 64 * 1024 && !lds_raised.count((const void *)fn)) {
             if (hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
@@ -771,6 +783,7 @@ int gemm_mfma_launch(const GemmDesc &d, int *limbs_a, int *limbs_b)
         fn<<<dim3((unsigned)blocks), dim3((unsigned)inst->threads), lds, 0>>>(p);
         g_last_pairs = kept_pairs_before(inst->na, inst->nb, inst->dmax, inst->na, 0);
         g_last_prepared = prep ? 1 : 0;
+        if (pipe_lds) g_pipe_calls++;
         {
             const hipError_t err = hipGetLastError();
             if (err != hipSuccess) {

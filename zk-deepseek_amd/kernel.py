@@ -76,6 +76,7 @@ lib.zk_gemm_guard_hits.restype = ctypes.c_long
 lib.zk_gemm_last_pairs.restype = ctypes.c_int
 lib.zk_gemm_grouped_mfma_calls.restype = ctypes.c_long
 lib.zk_gemm_grouped_streamed_calls.restype = ctypes.c_long
+lib.zk_gemm_pipe_calls.restype = ctypes.c_long
 lib.softmax_q19_scores.argtypes = [_vp] * 6 + [_ci] * 4 + [ctypes.c_longlong] * 2
 lib.silu_mul_q23.argtypes = [_vp] * 5 + [_ci] * 3
 lib.gate_route_q23.argtypes = [_vp] * 5 + [_ci] * 5
