@@ -1031,42 +1031,70 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm_split_finish_kernel(MfmaP
     const int tn = p.n_fastest ? rem % p.tiles_n : rem / p.tiles_m, tm = p.n_fastest ? rem / p.tiles_n : rem - tn * p.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
     const uint64_t rmask = p.shift ? ((1ull << p.shift) - 1) : 0;
+    const long qs = (long)(T / 64) * (WM * WN * 16);          // from one slice to the next
+    // the registers of this workgroup's share, RPER at a time with all their slices' loads under way together (one
+    // output at a time, a thread has `split` loads in flight and the launch lives on latency)
+    auto finish = [&](auto rper_tag) {
+        constexpr int RPER = decltype(rper_tag)::value;
 #pragma unroll
-    for (int a = 0; a < WM; a++)
+        for (int a = 0; a < WM; a++)
 #pragma unroll
-        for (int b = 0; b < WN; b++) {
-            const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
-            for (int r4 = 0; r4 < r_per; r4++) {
-                const int r = rq * r_per + r4;
-                const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) >= p.M) continue;      // never written
-                uint64_t lo = (uint64_t)p.init, hi = (uint64_t)(p.init >> 63);
-                const long q0 = ((long)tail_tile * p.split * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r;
-                const long qs = (long)(T / 64) * (WM * WN * 16);          // from one slice to the next
+            for (int b = 0; b < WN; b++) {
+                const int n = n0 + (wn * WN + b) * 32 + (lane & 31);
+                const int r0 = rq * RPER;
+                const long q0 = ((long)tail_tile * p.split * (T / 64) + wave) * (WM * WN * 16) + (a * WN + b) * 16 + r0;
+                uint64_t lo[RPER], hi[RPER];
+                bool live[RPER];
+#pragma unroll
+                for (int r4 = 0; r4 < RPER; r4++) {
+                    const int r = r0 + r4;
+                    lo[r4] = (uint64_t)p.init;
+                    hi[r4] = (uint64_t)(p.init >> 63);
+                    live[r4] = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + (r & 3) < p.M;      // (uniform over the wave; the others were never written)
+                }
                 if (p.part64) {
-                    uint64_t s = 0;
-#pragma unroll 16
-                    for (int sidx = 0; sidx < p.split; sidx++) s += p.partials[(q0 + sidx * qs) * 64 + lane];
-                    const uint64_t t = lo + s;
-                    hi += (uint64_t)((int64_t)s >> 63) + (t < lo ? 1 : 0);
-                    lo = t;
-                } else {
+                    uint64_t s[RPER];
+#pragma unroll
+                    for (int r4 = 0; r4 < RPER; r4++) s[r4] = 0;
 #pragma unroll 4
-                    for (int sidx = 0; sidx < p.split; sidx++) {
-                        const uint64_t plo = p.partials[(q0 + sidx * qs) * 128 + lane];
-                        const uint64_t phi = p.partials[(q0 + sidx * qs) * 128 + 64 + lane];
-                        const uint64_t t = lo + plo;
-                        hi += phi + (t < lo ? 1 : 0);
-                        lo = t;
+                    for (int sidx = 0; sidx < p.split; sidx++)
+#pragma unroll
+                        for (int r4 = 0; r4 < RPER; r4++)
+                            s[r4] += p.partials[(q0 + r4 + sidx * qs) * 64 + lane];      // (rows past M: slots nobody wrote, read and dropped)
+#pragma unroll
+                    for (int r4 = 0; r4 < RPER; r4++) {
+                        const uint64_t t = lo[r4] + s[r4];
+                        hi[r4] += (uint64_t)((int64_t)s[r4] >> 63) + (t < lo[r4] ? 1 : 0);
+                        lo[r4] = t;
+                    }
+                } else {
+#pragma unroll 2
+                    for (int sidx = 0; sidx < p.split; sidx++)
+#pragma unroll
+                        for (int r4 = 0; r4 < RPER; r4++)
+                        {
+                            const uint64_t plo = p.partials[(q0 + r4 + sidx * qs) * 128 + lane];
+                            const uint64_t phi = p.partials[(q0 + r4 + sidx * qs) * 128 + 64 + lane];
+                            const uint64_t t = lo[r4] + plo;
+                            hi[r4] += phi + (t < lo[r4] ? 1 : 0);
+                            lo[r4] = t;
+                        }
+                }
+#pragma unroll
+                for (int r4 = 0; r4 < RPER; r4++) {
+                    const int r = r0 + r4;
+                    const int m = m0 + (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (live[r4] && m < p.M && n < p.N) {
+                        const long o = (long)g * p.sC + (long)m * p.ldc + n;
+                        p.C[o] = (int64_t)(p.shift == 0 ? lo[r4] : ((lo[r4] >> p.shift) | (hi[r4] << (64 - p.shift))));
+                        if (p.R) p.R[o] = (int64_t)(lo[r4] & rmask);
                     }
                 }
-                if (m < p.M && n < p.N) {
-                    const long o = (long)g * p.sC + (long)m * p.ldc + n;
-                    p.C[o] = (int64_t)(p.shift == 0 ? lo : ((lo >> p.shift) | (hi << (64 - p.shift))));
-                    if (p.R) p.R[o] = (int64_t)(lo & rmask);
-                }
             }
-        }
+    };
+    if (r_per == 4) finish(std::integral_constant<int, 4>());
+    else if (r_per == 2) finish(std::integral_constant<int, 2>());
+    else finish(std::integral_constant<int, 1>());
 }
 
 // ---- kernel tables -------------------------------------------------------------------------------------
