@@ -25,3 +25,14 @@ def zk_tables():
     import json
     with open(os.path.join(ROOT, "tests", "golden", "zk_tables.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture(autouse=True)
+def _library_switches_at_their_defaults():
+    """a test that forces a GEMM path or lets softmax clobber its input must not decide what the next test runs on,
+    whatever the order: both switches are back at their defaults before every test (once the library is loaded)"""
+    k = sys.modules.get("kernel")
+    if k is not None and hasattr(k, "lib"):
+        k.lib.zk_gemm_set_path(0)
+        k.lib.zk_softmax_clobber_input(0)
+    yield
