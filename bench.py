@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20, help="untimed calls before the timed steps (at least; see SPIN_UP_MS)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,small,cold,cpu,calib (default gemm,extra,cpu; small = configs 1 and 2 of extra alone, cold = the calls on operands never seen alone)")
+    ap.add_argument("--only", default="", help="comma list of legs: gemm,extra,small,cold,prepared,cpu,calib (default gemm,extra,cpu; small = configs 1 and 2 of extra alone, cold = the calls on operands never seen alone, prepared = config 4 on prepared weights alone)")
     return ap.parse_args()
 
 
@@ -362,6 +362,7 @@ def run():
         nm = "gemm_config4_q31_x_int32"
         extra[nm] = gemm_leg(K, Am, Wm, 30, max(3, args.steps // 2), 1, samples, nm)
         del Am, Wm
+    if legs & {"extra", "prepared"}:
         # the headline shape with the weights prepared once as digit planes (zk_gemm_prepare_weights): what a model
         # with static weights gets; the one-time preparation is timed separately and is NOT part of `value`
         torch.cuda.synchronize()
@@ -371,6 +372,8 @@ def run():
         extra["gemm_config4_prepared_weights"] = gemm_leg(K, A, W, c, args.steps, 5, samples, "gemm_config4_prepared_weights", host=(A_h, W_h))
         extra["gemm_config4_prepared_weights"]["prepare_once_ms"] = prep_ms
         K.release_weights(W[0] if W.dim() == 3 else W)
+
+    if "extra" in legs:
         # other instruction path on the headline shape, for the comparison
         K.lib.zk_gemm_set_path(1 if path == 2 else 2)
         extra["gemm_config4_other_path"] = gemm_leg(K, A, W, c, 3, 1, samples, "gemm_config4_other_path", host=(A_h, W_h))
