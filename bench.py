@@ -825,6 +825,11 @@ def run():
     for nm, short in (("gemm_config2_w1_128x7168x2048", "gemm_config2_w1_us"), ("gemm_config2_w2_128x2048x7168", "gemm_config2_w2_us")):
         if nm in extra:
             flat[short] = extra[nm]["ms"] * 1e3
+    if "gemm_config4_prepared_weights" in extra:
+        # the headline product on weights prepared once (not `value`): its time and the same i8 operation count over it
+        e = extra["gemm_config4_prepared_weights"]
+        flat["gemm_config4_prepared_us"] = e["ms"] * 1e3
+        flat["gemm_config4_prepared_frac_mfma_peak"] = 2.0 * e["digit_pairs"] * e["macs"] / (e["ms"] * 1e-3) / 1e12 / I8_MFMA_PEAK_TOPS
     for nm in ("softmax_q19_1x1024x128x1024", "softmax_q19_1x4096x128x1024", "silu_q23_1x512x18432", "silu_q23_1x8192x18432",
                "sigmoid_q23_1x512x18432", "sigmoid_q23_1x8192x18432", "rmsnorm_fused_500x7168", "rmsnorm_fused_16384x7168"):
         if nm in extra:
@@ -871,7 +876,7 @@ def run():
     # the figures a reader wants first, once more at the very end of the line (a record that keeps only the tail of the
     # output still holds them)
     summary = {"value_gmacs": value, "ms_per_step": ms_per_step, "roofline_frac": roofline.get("frac"), "verified": bool(all_checked)}
-    summary.update({k: v for k, v in flat.items() if k.endswith(("_us", "_frac_hbm"))})
+    summary.update({k: v for k, v in flat.items() if k.endswith(("_us", "_frac_hbm", "_frac_mfma_peak"))})
     summary.update(cold)
     if cpu_baseline:
         summary["cpu_baseline_gmacs"] = cpu_baseline.get("value")
