@@ -4,6 +4,8 @@ circuits hold.  Nothing here launches a kernel."""
 import ctypes
 import os
 import re
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -150,3 +152,16 @@ def test_product_never_touches_the_checker():
     outside = src[:start] + src[end:]
     assert not re.search(r"^\s*(import|from)\s+oracle\b", outside, re.M)
     assert "oracle." not in outside
+
+
+def test_bench_refuses_more_than_one_gpu_and_defaults_to_one():
+    """the benchmark runs on one GPU: `--gpus 2` ends with a message and a non-zero status before anything touches a
+    device; with no flags it asks for one GPU and a step count that finishes in minutes"""
+    bench = os.path.join(ROOT, "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+    src = open(bench).read()
+    m = re.search(r'add_argument\("--gpus",[^)]*default=(\d+)', src)
+    assert m and int(m.group(1)) == 1
+    m = re.search(r'add_argument\("--steps",[^)]*default=(\d+)', src)
+    assert m and 1 <= int(m.group(1)) <= 1000
